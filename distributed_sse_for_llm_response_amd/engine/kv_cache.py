@@ -133,3 +133,27 @@ class MatrixStateCache(RecurrentStateCache):
         self.state = {r: torch.zeros(num_slots, *s, device=device, dtype=torch.float32) for r, (s, _, _) in shapes.items()}
         self.tail = {r: torch.zeros(num_slots, k - 1, c, device=device, dtype=torch.float32)
                      for r, (_, c, k) in shapes.items() if c > 0 and k > 1}
+
+
+class MixedKVCache:
+    """The paged caches of a design that has latent-attention runs AND key/value attention runs: a LatentKVCache for
+    the former and a PagedKVCache for the latter, over the same page ids, block tables and allocator (a page id means
+    the same page in every run of either kind)."""
+
+    def __init__(self, latent_widths: dict, kv_shapes: dict, num_blocks: int, device, dtype=torch.bfloat16,
+                 latent_transposed: dict | None = None, kv_transposed=()):
+        self.num_blocks = num_blocks
+        self.latent = LatentKVCache(latent_widths, num_blocks, device, dtype, transposed=latent_transposed)
+        self.paged = PagedKVCache(kv_shapes, num_blocks, device, dtype, transposed=kv_transposed)
+
+
+class ConvTailCache(RecurrentStateCache):
+    """Per-sequence tails of short causal convolutions that have no recurrence behind them, indexed by the decode slot
+    like RecurrentStateCache: per key the last taps - 1 inputs [slots, taps - 1, C] in fp32.  ``shapes`` maps a key
+    (for instance (run, sublayer)) -> (C, taps); keys with taps <= 1 hold nothing."""
+
+    def __init__(self, shapes: dict, num_slots: int, device):
+        self.num_slots = num_slots
+        self.state = {}
+        self.tail = {k: torch.zeros(num_slots, taps - 1, c, device=device, dtype=torch.float32)
+                     for k, (c, taps) in shapes.items() if taps > 1}

@@ -55,7 +55,8 @@ from .. import ops
 from ..models.muderax import LRU_DECAY_SCALE
 from ..models.surodra import UNIT_EPS
 from ..parallel.comm import TPComm
-from .kv_cache import PAGE, LatentKVCache, MatrixStateCache, PagedKVCache, RecurrentStateCache
+from .kv_cache import (PAGE, ConvTailCache, LatentKVCache, MatrixStateCache, MixedKVCache, PagedKVCache,
+                       RecurrentStateCache)
 from .model_runner import RunnerBase, _capture, batch_buckets
 from .weights import LayeredWeights
 
@@ -84,7 +85,10 @@ class LayeredRunner(RunnerBase):
         self._init_slots(max_batch, self.max_blocks, cfg.vocab_size, dev, self.comm)
         self.num_blocks = num_blocks
         self.prenorm = getattr(cfg, "family", "") == "surodra"   # pre-norm blocks with matrix-state mixers
-        if self.prenorm:
+        self.multistream = getattr(cfg, "family", "") == "dironex"  # pre-norm blocks on several residual streams
+        if self.multistream:
+            self._setup_streams()
+        elif self.prenorm:
             self._setup_prenorm()
         else:
             self._setup_sandwich()
@@ -137,6 +141,9 @@ class LayeredRunner(RunnerBase):
         el = dict(device=dev, dtype=self.dtype)
         W = cfg.width
         d = {"resid": torch.zeros(M, W, **f32), "xb": torch.zeros(M, W, **el), "y": torch.zeros(M, W, **f32)}
+        if self.multistream:
+            d.update(self._stream_buffers(M))
+            return d
         if self.prenorm:
             d.update(self._prenorm_buffers(M))
             return d
@@ -261,6 +268,9 @@ class LayeredRunner(RunnerBase):
         portions), each with its own metadata (block tables bt, q_start qs, q_len ql, ctx_len ctx, state slots ss,
         attention work items ws / wt of qt rows).  trace (a list) receives a copy of the stream after every layer."""
         cfg, eps = self.cfg, self.cfg.eps
+        if self.multistream:
+            self._stream_layers(M, d, ids, pos, slots, groups, trace)
+            return
         ops.embed_rows(ids, self.w.embed, d["resid"], d["xb"])
         if self.prenorm:
             self._prenorm_layers(M, d, ids, pos, slots, groups, trace)
@@ -284,7 +294,11 @@ class LayeredRunner(RunnerBase):
         self._head(rows, xn, logits)
 
     def _head(self, resid, xn, logits) -> None:
-        if self.prenorm:
+        if self.multistream:  # resid holds the sum of the streams: one stream with weight 1 through the RMS norm
+            ops.stream_mix(None, 1, 0.0, resid.unsqueeze(1), in_w=self.w.ones[:1], norm_w=self.w.final_norm,
+                           eps=self.cfg.eps, h=xn)
+            self._lin(xn, self.w.head, self.w.head_t, logits)
+        elif self.prenorm:
             n, cfg = self.w.final_norm, self.cfg
             ops.stream_step(None, 0.0, resid, None, None, None, n.alpha, n.w, n.b, xn)
             self._lin(xn, self.w.head, self.w.head_t, logits)
@@ -459,6 +473,202 @@ class LayeredRunner(RunnerBase):
         self._scan_out(ri, None, big[:, 2 * H * D + H * V:], H, V, M, d, q, k, v, Lw.decay, None, groups, 1.0, Lw.o,
                        Lw.o_t, d["y"])
 
+    # ------------------------------------------------------------------ pre-norm designs on several residual streams
+    def _setup_streams(self) -> None:
+        """Caches and state of a design on several residual streams, keyed by layer RUN: latent rows for the
+        latent-attention runs, keys and values for the windowed-attention runs (same pages and block tables), and the
+        tails of the input convolutions of both sublayers of every run."""
+        cfg, dev = self.cfg, self.device
+        self.runs = cfg.runs()
+        lat, kv, tails, self._rope = {}, {}, {}, {}
+        for r in self.runs:
+            L, m = cfg.layers[r.layer], cfg.layers[r.layer].mixer
+            if L.kind == "latent_attention":
+                lat[r.index] = m
+                key = (m.rot, m.rot_dim)
+                if key not in self._rope:
+                    self._rope[key] = m.rot.table(self.max_model_len + 1, m.rot_dim, dev)
+            else:
+                kv[r.index] = (m.kv_heads, m.dim, m.vdim)
+            tails[(r.index, 1)] = (cfg.width, cfg.canon_taps)
+            if L.mlp is not None:
+                tails[(r.index, 2)] = (cfg.width, cfg.canon_taps)
+        lflash = {r: m.kv_rank for r, m in lat.items() if ops.latent_flash_ok(self.dtype, m.kv_rank, m.rot_dim)}
+        kflash = [r for r, (_, dm, v) in kv.items() if ops.sink_flash_ok(self.dtype, dm, v)]
+        self.kv = MixedKVCache({r: m.kv_rank + m.rot_dim for r, m in lat.items()}, kv, self.num_blocks, dev, self.dtype,
+                               latent_transposed=lflash, kv_transposed=kflash)
+        self.state = ConvTailCache(tails, self.max_batch, dev)
+        words = max((ops.latent_flash_part_floats(self.max_batch, m.heads, 16, 16, m.kv_rank) for r, m in lat.items()
+                     if r in lflash), default=0)
+        self._flash_part = torch.zeros(max(1, words), device=dev, dtype=torch.float32)
+
+    def _stream_buffers(self, M: int) -> dict:
+        """Scratch of a step of M rows, each sized for the widest layer: `streams` the residual copies, `hn` a
+        sublayer's normed input and `hc` it after the input convolution (fp32), `big` the fused projection's fp32
+        output, `cq` the normed query latent, `q` / `qabs` / `lat` the latent attention's operands, `o` a mixer's
+        heads in fp32, `ao` them in the element type (the output projection's input), `up` / `h` the dense
+        feed-forward's hidden row, and the routed experts' lists."""
+        cfg, dev = self.cfg, self.device
+        f32 = dict(device=dev, dtype=torch.float32)
+        el = dict(device=dev, dtype=self.dtype)
+        W = cfg.width
+        big = cq = q = qabs = o = ff = qa = 1
+        moe = []
+        for i, L in enumerate(cfg.layers):
+            m = L.mixer
+            big = max(big, self.w.layers[i].mix.n_big)
+            if L.kind == "latent_attention":
+                cq, q = max(cq, m.q_rank), max(q, m.heads * (m.dim + m.rot_dim))
+                qabs, o = max(qabs, m.heads * m.kv_rank), max(o, m.heads * m.vdim)
+            else:
+                qa, o = max(qa, m.heads * m.dim), max(o, m.heads * m.vdim)
+            if L.mlp is not None:
+                if hasattr(L.mlp, "experts"):
+                    moe.append(L.mlp)
+                else:
+                    ff = max(ff, L.mlp.ff)
+        d = {"streams": torch.zeros(M, cfg.num_streams, W, **f32), "hn": torch.zeros(M, W, **f32),
+             "hc": torch.zeros(M, W, **f32), "big": torch.zeros(M * big, **f32), "cq": torch.zeros(M * cq, **el),
+             "q": torch.zeros(M * q, **el), "qabs": torch.zeros(M * qabs, **f32), "lat": torch.zeros(M * qabs, **el),
+             "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32), "ao": torch.zeros(M * o, **el),
+             "up": torch.zeros(M * ff, **f32), "h": torch.zeros(M * ff, **el)}
+        if moe:
+            top = max(f.top for f in moe)
+            tiles = -(-M * top // 64) + max(f.experts for f in moe) + 2
+            ldh = -(-max(f.ff for f in moe) // 8) * 8
+            d.update({"tki": torch.zeros(M * top, device=dev, dtype=torch.int32), "tkw": torch.zeros(M * top, **f32),
+                      "mo_z": torch.zeros(M * max(f.experts for f in moe), **f32),
+                      "mo_sorted": torch.zeros(tiles * 64, device=dev, dtype=torch.int32),
+                      "mo_tile": torch.zeros(tiles, device=dev, dtype=torch.int32),
+                      "mo_n": torch.zeros(1, device=dev, dtype=torch.int32), "mo_h": torch.zeros(M * top, ldh, **el),
+                      "mo_o": torch.zeros(M * top * W, **f32)})
+        return d
+
+    def _stream_layers(self, M: int, d: dict, ids, pos, slots, groups: list, trace: list | None) -> None:
+        """Every layer run over M packed rows.  Between sublayers ONE stream_mix writes the finished sublayer's output
+        into all streams (through its mix matrix and output weights, times the residual multiplier), forms the next
+        sublayer's input from them and RMS-norms it; the first one also fills the streams with the scaled embedding.
+        The input convolution then continues each sequence's tail.  At the end d["resid"] holds the sum of the streams
+        (what the head's norm reads)."""
+        cfg, w = self.cfg, self.w
+        mult, eps, x = cfg.residual_mult, cfg.eps, d["streams"]
+        prev = None  # (output rows, parts per row, stream weights) of the sublayer that is not written back yet
+        first = True
+        for run in self.runs:
+            L, Lw = cfg.layers[run.layer], w.layers[run.layer]
+            for sub, hc in ((1, Lw.hc1), (2, Lw.hc2)):
+                if hc is None:
+                    continue
+                y, nsum, pw = prev if prev else (None, 1, None)
+                conv = hc.canon is not None and hc.canon.shape[1] > 0
+                ops.stream_mix(y, nsum, mult, x, ids if first else None, w.embed if first else None, cfg.embed_scale,
+                               pw.outw if pw else None, pw.mix if pw else None, hc.inw, hc.norm, eps,
+                               d["hn"] if conv else d["xb"])
+                first = False
+                if conv:
+                    for g in groups:
+                        ops.conv_state(d["hn"], hc.canon, None, self.state.tail.get((run.index, sub)), g["qs"], g["ql"],
+                                       g["ctx"], g["ss"], d["hc"], d["xb"], None, 2)
+                if sub == 1:
+                    getattr(self, "_" + L.kind + "_streams")(run.index, L.mixer, Lw.mix, M, d, pos, slots, groups)
+                    prev = (d["y"], 1, hc)
+                elif hasattr(L.mlp, "experts"):
+                    prev = self._routed_ff(L.mlp, Lw.mlp, M, d) + (hc,)
+                else:
+                    self._act_ff(L.mlp, Lw.mlp, M, d)
+                    prev = (d["y"], 1, hc)
+            if trace is not None:
+                y, nsum, pw = prev
+                ops.stream_mix(y, nsum, mult, x, out_w=pw.outw, mix=pw.mix, total=d["resid"])
+                prev = None
+                trace.append(d["resid"].clone())
+        y, nsum, pw = prev if prev else (None, 1, None)
+        ops.stream_mix(y, nsum, mult, x, ids if first else None, w.embed if first else None, cfg.embed_scale,
+                       pw.outw if pw else None, pw.mix if pw else None, total=d["resid"])
+
+    def _latent_attention_streams(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        """Latent attention with a query latent and a sigmoid output gate: ONE fused GEMM [dq | dkv | g] (fp32 out) ->
+        RMS norm of the query latent -> query up-projection; latent_kv_write (norm + rotation + cache row) from the
+        dkv columns; folded attention over this run's latent pages; per-head value up-projection (fp32) times
+        sigmoid(g) -> output GEMM."""
+        H, dn, dr, rk, dv, qr = m.heads, m.dim, m.rot_dim, m.kv_rank, m.vdim, m.q_rank
+        rope = self._rope[(m.rot, m.rot_dim)]
+        cache, vt = self.kv.latent[ri], self.kv.latent.vt.get(ri)
+        big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
+        cq = d["cq"][:M * qr].view(M, qr)
+        q = d["q"][:M * H * (dn + dr)].view(M, H, dn + dr)
+        qabs = d["qabs"][:M * H * rk].view(M, H, rk)
+        lat = d["lat"][:M * H * rk].view(M, H, rk)
+        o = d["o"][:M * H * dv].view(M, H, dv)
+        ao = d["ao"][:M * H * dv].view(M, H * dv)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        ops.norm_rope_rows(big[:, :qr].unsqueeze(1), Lw.dq_norm, pos, None, cq.unsqueeze(1), None, 1, self.cfg.eps, 1.0)
+        self._lin(cq, Lw.uq, Lw.uq_t, q.view(M, H * (dn + dr)))
+        ops.latent_kv_write(big[:, qr:qr + rk + dr], Lw.dkv_norm, pos, slots, rope, cache, self.cfg.eps, vt)
+        ops.gemm_rm(q[:, :, :dn].permute(1, 0, 2), Lw.uk_t, qabs.permute(1, 0, 2))
+        for g in groups:
+            if vt is not None:
+                if g["qt"] == 1:
+                    np_ = self._decode_parts(g["ws"].numel(), H, m.window)
+                    ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope,
+                                         lat, m.window, m.scale, 1, vt, 16, self._flash_part if np_ > 1 else None, np_)
+                else:
+                    ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["fs"], g["ft"], rope,
+                                         lat, m.window, m.scale, FLASH_ROWS_TILE, vt, 16 // FLASH_ROWS_TILE)
+            else:
+                ops.latent_attention(q, qabs, cache, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], rope, lat,
+                                     m.window, m.scale, g["qt"])
+        ops.gemm_rm(lat.permute(1, 0, 2), Lw.uv, o.permute(1, 0, 2))
+        ops.act_rows(o.view(M, H * dv), ao, 0, None, big[:, qr + rk + dr:qr + rk + dr + H * dv])
+        self._lin(ao, Lw.o, Lw.o_t, d["y"])
+
+    def _attention_streams(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        """Sliding-window attention with grouped key/value heads and per-head RMS norms on q and k, no rotation: ONE
+        fused GEMM [q | k | v] -> norm rows (q to a buffer, k and v straight into this run's pages) -> attention over
+        the window (MFMA form where the head widths allow it) -> output GEMM."""
+        H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
+        big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        kc, vc, vt = self.kv.paged.k[ri], self.kv.paged.v[ri], self.kv.paged.vt.get(ri)
+        qa = d["qa"][:M * H * D].view(M, H, D)
+        eps = self.cfg.eps
+        ops.norm_rope_rows(self._cols(big, 0, H, D), Lw.q_norm, pos, None, qa, None, 3, eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, H * D, G, D), Lw.k_norm, pos, None, kc, slots, 3, eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, (H + G) * D, G, V), None, pos, None, vc, slots, 0, 0.0, 1.0, vt)
+        ao = d["ao"][:M * H * V].view(M, H, V)
+        for g in groups:
+            if vt is not None and g["qt"] > 1:
+                ops.sink_attention(qa, kc, vc, g["bt"], g["qs"], g["ql"], g["ctx"], g["hs"], g["ht"], None, None, ao,
+                                   m.window, m.scale, SINK_ROWS_TILE, vt)
+            elif vt is not None and V <= ops.layers.SINK_SPLIT_MAX_V:
+                ops.sink_attention(qa, kc, vc, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], None, None, ao,
+                                   m.window, m.scale, SINK_ROWS_TILE, vt, True)
+            else:
+                ops.sink_attention(qa, kc, vc, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], None, None, ao,
+                                   m.window, m.scale, g["qt"])
+        self._lin(ao.view(M, H * V), Lw.o, Lw.o_t, d["y"])
+
+    def _act_ff(self, f, Fw, M: int, d: dict) -> None:
+        """Dense feed-forward: up GEMM (fp32) -> xIELU -> down GEMM."""
+        up = d["up"][:M * f.ff].view(M, f.ff)
+        h = d["h"][:M * f.ff].view(M, f.ff)
+        self._lin(d["xb"], Fw.up, Fw.up_t, up)
+        ops.act_rows(up, h, 1, Fw.act)
+        self._lin(h, Fw.down, Fw.down_t, d["y"])
+
+    def _routed_ff(self, f, Fw, M: int, d: dict):
+        """Router GEMM (fp32 logits) -> group-limited sigmoid routing -> grouped squared-ReLU experts; returns
+        (per-slot outputs [M * top, W] fp32, top): the stream step that follows sums them."""
+        tki = d["tki"][:M * f.top].view(M, f.top)
+        tkw = d["tkw"][:M * f.top].view(M, f.top)
+        o = d["mo_o"][:M * f.top * self.cfg.width].view(M * f.top, self.cfg.width)
+        z = d["mo_z"][:M * f.experts].view(M, f.experts)
+        ops.gemm_rm(d["xb"], Fw.router, z)
+        ops.moe_route(z, Fw.correction, tki, tkw, f.groups, f.keep, f.scale)
+        ops.moe_grouped(d["xb"], tki, tkw, None, Fw.up, Fw.down, None, None, None, d["mo_sorted"], d["mo_tile"],
+                        d["mo_n"], d["mo_h"], o)
+        return o, f.top
+
     # ------------------------------------------------------------------ decode
     def _decode_group(self, B: int) -> dict:
         r = slice(0, B)
@@ -471,7 +681,7 @@ class LayeredRunner(RunnerBase):
         r = slice(0, B)
         ops.decode_prep(self.active[r], self.positions[r], self.block_tables[r], self.slots[r], self.ctx_len[r],
                         self.q_len[r], self.kv.num_blocks)
-        d = {k: (v[:B] if k in ("resid", "xb", "y", "y2") else v) for k, v in self._dec.items()}
+        d = {k: (v[:B] if k in ("resid", "xb", "y", "y2", "streams", "hn", "hc") else v) for k, v in self._dec.items()}
         self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
         self._head(d["resid"], self._dec["xb"][:B], self.logits[r])
         self._sample_commit(B)

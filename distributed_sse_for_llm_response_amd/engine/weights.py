@@ -259,6 +259,7 @@ class LayeredWeights:
     tp_size: int = 1
     head_t: torch.Tensor = None  # the head in the tiled layout when its shape fits (head then None)
     step: torch.Tensor = None    # [passes, W] fp32: the vector added before each pass of a looped span (or None)
+    ones: torch.Tensor = None    # [streams] fp32 ones of a design on several residual streams (or None)
 
     @property
     def vocab_local(self) -> int:
@@ -281,7 +282,7 @@ class LayeredWeights:
 
         for L in self.layers:
             n += size(L)
-        return n + sum(size(t) for t in (self.embed, self.final_norm, self.head, self.head_t, self.step))
+        return n + sum(size(t) for t in (self.embed, self.final_norm, self.head, self.head_t, self.step, self.ones))
 
 
 TILED_MIN = 1024  # smallest N and K that go to the tiled-layout GEMMs
@@ -509,3 +510,168 @@ def load_surodra_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> Laye
     for f in sorted(Path(path).glob("*.safetensors")):
         tensors.update(load_file(str(f)))
     return convert_surodra(cfg, tensors, device=device, dtype=dtype)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Designs on several residual streams (models/dironex.py).  Projections that read the same input are ONE weight, as for
+# the other pre-norm family; stream weights, norm gains, router corrections and activation constants are fp32 in both
+# element types.  The latent attention kernels rotate interleaved pairs (2i, 2i + 1); this family pairs coordinate i
+# with i + dims / 2, so the rows of the two projections that make the rotated parts (the query up-projection's rotated
+# rows of every head, the down-projection's shared key rows) are permuted at load: pair i lands on (2i, 2i + 1) of both
+# operands, a scalar product is the same under a common permutation, and nothing else reads those coordinates.
+@dataclass
+class StreamWeights:
+    inw: torch.Tensor        # [S] fp32: the sublayer's input is sum_s inw[s] x_s
+    outw: torch.Tensor       # [S] fp32: stream t receives mult * outw[t] * y
+    mix: torch.Tensor        # [S, S] fp32, [from, to]
+    norm: torch.Tensor       # [W] fp32 gain of the RMS norm on the input
+    canon: torch.Tensor      # [W, taps] element type, or None
+
+
+@dataclass
+class GatedLatentWeights:
+    big: torch.Tensor        # rows [dq (q_rank) | dkv (rk + dr, rotated rows interleaved) | g (H dv) | zero rows] x W
+    n_big: int
+    dq_norm: torch.Tensor    # [q_rank] fp32
+    uq: torch.Tensor         # [H (dn + dr), q_rank], rotated rows of every head interleaved
+    dkv_norm: torch.Tensor   # [rk] element type
+    uk_t: torch.Tensor       # [H, rk, dn]
+    uv: torch.Tensor         # [H, dv, rk]
+    o: torch.Tensor          # [W, H dv]
+    big_t: torch.Tensor = None
+    uq_t: torch.Tensor = None
+    o_t: torch.Tensor = None
+
+
+@dataclass
+class WindowAttentionWeights:
+    big: torch.Tensor        # rows [q (H D) | k (G D) | v (G V) | zero rows] x W
+    n_big: int
+    q_norm: torch.Tensor     # [D] fp32
+    k_norm: torch.Tensor     # [D] fp32
+    o: torch.Tensor
+    big_t: torch.Tensor = None
+    o_t: torch.Tensor = None
+
+
+@dataclass
+class ActFfWeights:
+    up: torch.Tensor         # [F, W]
+    down: torch.Tensor       # [W, F]
+    act: torch.Tensor        # [2] fp32: (softplus(p), 1/2 + softplus(q)) of the xIELU activation
+    up_t: torch.Tensor = None
+    down_t: torch.Tensor = None
+
+
+@dataclass
+class RoutedFfWeights:
+    router: torch.Tensor     # [E, W]
+    correction: torch.Tensor  # [E] fp32
+    up: torch.Tensor         # [E, F, W]
+    down: torch.Tensor       # [E, W, F]
+
+
+@dataclass
+class StreamLayer:
+    hc1: StreamWeights
+    mix: object
+    hc2: StreamWeights = None
+    mlp: object = None
+
+
+def interleave_half_pairs(width: int, dims: int) -> torch.Tensor:
+    """Index list that moves a rotate-half pair (i, i + dims / 2) of a `width`-wide rotated part to (2i, 2i + 1); the
+    coordinates from `dims` on keep their place."""
+    idx = torch.arange(width)
+    half = dims // 2
+    idx[0:dims:2] = torch.arange(half)
+    idx[1:dims:2] = torch.arange(half) + half
+    return idx
+
+
+@torch.no_grad()
+def convert_dironex(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """Checkpoint tensors {name: tensor} (models/dironex.py tensor_shapes) -> the engine's grouped layout in `dtype`."""
+    from ..models.dironex import DenseSpec, tensor_shapes
+
+    for name, shape in tensor_shapes(cfg).items():
+        if name not in tensors:
+            raise KeyError(f"checkpoint lacks tensor {name!r}")
+        if tuple(tensors[name].shape) != tuple(shape):
+            raise ValueError(f"tensor {name!r} has shape {tuple(tensors[name].shape)}, the configuration says {shape}")
+
+    def t(name):
+        return tensors[name].to(device=device, dtype=dtype).contiguous()
+
+    def f(name):
+        return tensors[name].to(device=device, dtype=torch.float32).contiguous()
+
+    def cat(*parts):
+        w = torch.cat(parts, dim=0)
+        if w.shape[0] >= TILED_MIN and w.shape[0] % 128:
+            w = torch.cat([w, w.new_zeros(128 - w.shape[0] % 128, w.shape[1])], dim=0)
+        return w.contiguous()
+
+    S, W = cfg.num_streams, cfg.width
+
+    def stream(p, q):
+        if cfg.streams > 0:
+            inw, outw, mix = f(f"{p}hc{q}.in"), f(f"{p}hc{q}.out"), f(f"{p}hc{q}.mix")
+        else:
+            inw, outw, mix = (torch.ones(n, device=device, dtype=torch.float32) for n in ((1,), (1,), (1, 1)))
+        return StreamWeights(inw=inw, outw=outw, mix=mix, norm=f(f"{p}norm{q}"),
+                             canon=t(f"{p}canon{q}") if cfg.canon_taps > 0 else None)
+
+    layers = []
+    for i, L in enumerate(cfg.layers):
+        p, m = f"l{i}.", L.mixer
+        if L.kind == "latent_attention":
+            H, dn, dr, rk = m.heads, m.dim, m.rot_dim, m.kv_rank
+            perm = interleave_half_pairs(dr, m.rot.dims).to(device)
+            dkv = t(p + "mix.dkv")
+            dkv = torch.cat([dkv[:rk], dkv[rk:][perm]], dim=0)
+            uq = t(p + "mix.uq").view(H, dn + dr, m.q_rank)
+            uq = torch.cat([uq[:, :dn], uq[:, dn:][:, perm]], dim=1).reshape(H * (dn + dr), m.q_rank).contiguous()
+            big = cat(t(p + "mix.dq"), dkv, t(p + "mix.g"))
+            mix = GatedLatentWeights(
+                big=big, n_big=big.shape[0], dq_norm=f(p + "mix.dq.norm"), uq=uq, dkv_norm=t(p + "mix.dkv.norm"),
+                uk_t=t(p + "mix.uk").view(H, dn, rk).transpose(1, 2).contiguous(),
+                uv=t(p + "mix.uv").view(H, m.vdim, rk).contiguous(), o=t(p + "mix.o"))
+            _tile_fields(mix, ("big", "uq", "o"))
+        else:
+            big = cat(t(p + "mix.q"), t(p + "mix.k"), t(p + "mix.v"))
+            mix = WindowAttentionWeights(big=big, n_big=big.shape[0], q_norm=f(p + "mix.q.norm"),
+                                         k_norm=f(p + "mix.k.norm"), o=t(p + "mix.o"))
+            _tile_fields(mix, ("big", "o"))
+        layer = StreamLayer(hc1=stream(p, "1"), mix=mix)
+        fs = L.mlp
+        if fs is not None:
+            layer.hc2 = stream(p, "2")
+            if isinstance(fs, DenseSpec):
+                pq = tensors[p + "mlp.act"].to(torch.float64)
+                sp = torch.nn.functional.softplus(pq)
+                act = torch.stack([sp[0], 0.5 + sp[1]]).to(device=device, dtype=torch.float32)
+                layer.mlp = ActFfWeights(up=t(p + "mlp.up"), down=t(p + "mlp.down"), act=act)
+                _tile_fields(layer.mlp, ("up", "down"))
+            else:
+                stack = lambda leaf: torch.stack([t(f"{p}mlp.e{e}.{leaf}") for e in range(fs.experts)]).contiguous()  # noqa: E731
+                layer.mlp = RoutedFfWeights(router=t(p + "mlp.router"), correction=f(p + "mlp.correction"),
+                                            up=stack("up"), down=stack("down"))
+        layers.append(layer)
+    out = LayeredWeights(cfg=cfg, embed=t("embed"), layers=layers, final_norm=f("final.norm"), head=t("head"),
+                         dtype=dtype)
+    out.ones = torch.ones(S, device=device, dtype=torch.float32)   # the head reads the plain sum of the streams
+    _tile_fields(out, ("head",))
+    return out
+
+
+def load_dironex_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """``*.safetensors`` of a checkpoint directory -> the engine's layout (the loader executes nothing from them)."""
+    from pathlib import Path
+
+    from safetensors.torch import load_file
+
+    tensors = {}
+    for f in sorted(Path(path).glob("*.safetensors")):
+        tensors.update(load_file(str(f)))
+    return convert_dironex(cfg, tensors, device=device, dtype=dtype)

@@ -82,7 +82,8 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
 def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None, act: int = 0):
     """Per-channel causal convolution continued from each sequence's slot tail (and the tail's update); in_bias is
     added to every input (the bias of the projection that made `inp`).  `inp` may be a column slice of a wider fp32
-    buffer; bias and out_b (the output once more in the element type) may be None; act 1 applies SiLU to the output."""
+    buffer; bias and out_b (the output once more in the element type) may be None; act 1 applies SiLU to the output, act 2
+    adds the row's own input to it (inp + conv(inp))."""
     if _hip(inp):
         torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias, act)
     else:
@@ -128,8 +129,9 @@ def moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out):
 
 def moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, sorted_ids, tile_expert, num_tiles, h, o):
     """Grouped form of the routed experts: rows sorted by expert, 16-row MFMA tiles of one expert each.  o [M · S, W]
-    (fp32) = weight · expert output per (row, slot), S = top (+ 1: the shared expert's slot); scalar_norm(nsum=S) sums
-    them.  sorted_ids / tile_expert / num_tiles / h are scratch."""
+    (fp32) = weight · expert output per (row, slot), S = top (+ 1: the shared expert's slot); the norm or stream step
+    that follows sums them (nsum=S).  gate None: experts without a gate, down(relu(up x)^2).  sorted_ids / tile_expert /
+    num_tiles / h are scratch."""
     if _hip(x):
         torch.ops.dsse.moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, sorted_ids, tile_expert,
                                    num_tiles, h, o)
@@ -159,7 +161,8 @@ def gated_act(gu, h, kind: int = 1):
 
 def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind: int, eps: float, scale: float = 1.0, out_t=None):
     """Rows x [T, heads, D] (fp32, may be a column slice of a wider buffer) -> out rows out_rows[t] (or t) in out's
-    type: an optional norm (1: RMS over the whole row times norm_w; 2: unit vector per head), the rotate-half rotation
+    type: an optional norm (1: RMS over the whole row times norm_w [heads * D]; 2: unit vector per head; 3: RMS per head
+    times norm_w [D], one gain vector for all heads), the rotate-half rotation
     of the leading 2 * rope.shape[1] coordinates (rope [positions, dims / 2, 2] or None), times scale.  With out_rows =
     cache rows this writes keys or values straight into their pages [pages, 32, heads, D]; out_t (optional,
     [pages, heads, D, 32]) receives them once more in transposed pages (the MFMA attention's value operand)."""
@@ -287,3 +290,38 @@ def logit_cap(logits, scale: float, cap: float):
         torch.ops.dsse.logit_cap(logits, scale, cap)
     else:
         lref.logit_cap(logits, scale, cap)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Designs on several residual streams with routed squared-ReLU experts.
+def stream_mix(y, nsum: int, mult: float, streams, ids=None, embed=None, embed_scale: float = 1.0, out_w=None, mix=None,
+               in_w=None, norm_w=None, eps: float = 0.0, h=None, total=None):
+    """One pass over the S residual streams [M, S, W] (fp32) of each row, between two sublayers.  embed given: every
+    stream = embed[ids] * embed_scale (a model's first step).  y given ([M * nsum, W] fp32, a row's nsum consecutive
+    parts are summed first): x_t = sum_s mix[s, t] x_s + mult * out_w[t] * y for all streams at once.  in_w given: the
+    next sublayer's input u = sum_s in_w[s] x_s, RMS-normed with the gain norm_w [W], into h (fp32 or the element
+    type).  total given: the sum of the streams (fp32).  out_w, in_w [S], mix [S, S] and norm_w are fp32."""
+    if _hip(streams):
+        torch.ops.dsse.stream_mix(y, nsum, mult, streams, ids, embed, embed_scale, out_w, mix, in_w, norm_w, eps, h, total)
+    else:
+        lref.stream_mix(y, nsum, mult, streams, ids, embed, embed_scale, out_w, mix, in_w, norm_w, eps, h, total)
+
+
+def act_rows(x, out, kind: int, params=None, gate=None):
+    """out [M, F] (fp32 or the element type) = act(x) * sigmoid(gate) for fp32 x and gate (column slices are fine; gate
+    may be None).  kind 0: identity; 1: xIELU, a_p z^2 + z / 2 for z > 0 else a_n (e^z - 1 - z) + z / 2 with
+    params = fp32 (a_p, a_n); 2: relu(z)^2."""
+    if _hip(x):
+        torch.ops.dsse.act_rows(x, out, kind, params, gate)
+    else:
+        lref.act_rows(x, out, kind, params, gate)
+
+
+def moe_route(z, correction, topk_idx, topk_w, groups: int, keep: int, scale: float):
+    """Group-limited sigmoid routing from fp32 logits z [M, E]: choice scores sigmoid(z) + correction [E]; of `groups`
+    equal groups of neighbouring experts only the `keep` with the largest sum of their two best choice scores are
+    eligible; the top experts by choice score get the weights sigmoid(z) / (their sum + 1e-20) * scale."""
+    if _hip(z):
+        torch.ops.dsse.moe_route(z, correction, topk_idx, topk_w, groups, keep, scale)
+    else:
+        lref.moe_route(z, correction, topk_idx, topk_w, groups, keep, scale)

@@ -105,7 +105,8 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
 
 
 def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None, act=0):
-    """inp may be a column slice of a wider buffer; act 1: SiLU on the output (the tail keeps raw inputs)."""
+    """inp may be a column slice of a wider buffer; act 1: SiLU on the output (the tail keeps raw inputs); act 2: the
+    row's own input is added to its output (inp + conv(inp))."""
     K = taps.shape[1]
     tp = taps.float()
     ib = 0.0 if in_bias is None else in_bias.float()
@@ -122,6 +123,8 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
             y = y + seq[k:k + ql] * tp[:, k]
         if act == 1:
             y = torch.nn.functional.silu(y)
+        elif act == 2:
+            y = y + seq[K - 1:]
         out[r0:r0 + ql] = y
         if out_b is not None:
             out_b[r0:r0 + ql] = y.to(out_b.dtype)
@@ -189,19 +192,22 @@ def moe_ffn(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, out):
 
 
 def moe_grouped(x, topk_idx, topk_w, gate, up, down, sgate, sup, sdown, o):
-    """o [M * S, W]: slot k < top of row r = weight * expert output, slot `top` = the shared expert."""
+    """o [M * S, W]: slot k < top of row r = weight * expert output, slot `top` = the shared expert.  gate None: the
+    experts are down(relu(up x)^2), without a gate."""
     xf = x.float()
     M, top = topk_idx.shape
     S = top + (1 if sgate is not None else 0)
     ov = o.view(M, S, -1)
 
     def ffn(h, g, u, d):
+        if g is None:
+            return torch.relu(h @ u.float().t()).pow(2).to(x.dtype).float() @ d.float().t()
         return (torch.nn.functional.silu(h @ g.float().t()) * (h @ u.float().t())) @ d.float().t()
 
-    for e in range(gate.shape[0]):
+    for e in range(up.shape[0]):
         rows, ks = torch.nonzero(topk_idx == e, as_tuple=True)
         if rows.numel():
-            ov[rows, ks] = ffn(xf[rows], gate[e], up[e], down[e]) * topk_w[rows, ks].unsqueeze(-1)
+            ov[rows, ks] = ffn(xf[rows], None if gate is None else gate[e], up[e], down[e]) * topk_w[rows, ks].unsqueeze(-1)
     if sgate is not None:
         ov[:, top] = ffn(xf, sgate, sup, sdown)
 
@@ -245,6 +251,7 @@ def rotate_half_rows(v, cs, dims):
 def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, scale, out_t=None):
     """x [T, heads, D] fp32 -> out rows (out_rows[t], or t) as [heads, D] in out's type.  norm_kind 1: RMS norm over
     the whole row (all heads at once) times norm_w [heads * D]; 2: every head divided by sqrt(sum of squares + eps);
+    3: RMS norm per head times norm_w [D] (one gain vector for all heads);
     then the rotate-half rotation of the leading 2 * rope.shape[1] coordinates at positions[t]; then times scale.
     Rows whose out_rows entry is negative are skipped."""
     T, nh, D = x.shape
@@ -254,6 +261,8 @@ def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, sc
         v = (flat / torch.sqrt(flat.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()).view(T, nh, D)
     elif norm_kind == 2:
         v = v / torch.sqrt(v.pow(2).sum(-1, keepdim=True) + eps)
+    elif norm_kind == 3:
+        v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
     if rope is not None and rope.shape[1] > 0:
         pos = positions[:T].long().clamp(0, rope.shape[0] - 1)
         v = rotate_half_rows(v, rope[pos], 2 * rope.shape[1])
@@ -365,3 +374,58 @@ def logit_cap(logits, scale, cap):
     logits.mul_(scale)
     if cap > 0:
         logits.copy_(cap * torch.tanh(logits / cap))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Designs on several residual streams with routed squared-ReLU experts (models/dironex.py)
+def stream_mix(y, nsum, mult, streams, ids, embed, embed_scale, out_w, mix, in_w, norm_w, eps, h, total):
+    """streams [M, S, W] fp32.  embed given: every stream = embed[ids] * embed_scale.  y given ([M * nsum, W], a row's
+    nsum consecutive parts summed first): x_t = sum_s mix[s, t] x_s + mult * out_w[t] * y, all streams at once from the
+    old ones.  in_w given: u = sum_s in_w[s] x_s and h = u / rms(u) * norm_w in h's type.  total given: sum_s x_s."""
+    M, S, W = streams.shape
+    if embed is not None:
+        idx = ids[:M].long()
+        idx = torch.where((idx >= 0) & (idx < embed.shape[0]), idx, torch.zeros_like(idx))
+        streams.copy_((embed[idx].float() * embed_scale)[:, None, :].expand(M, S, W))
+    if y is not None:
+        ys = y.float().view(M, nsum, W).sum(1)
+        streams.copy_(torch.einsum("st,msw->mtw", mix.float(), streams) + mult * out_w.float()[None, :, None] * ys[:, None])
+    if in_w is not None:
+        u = torch.einsum("s,msw->mw", in_w.float(), streams)
+        h.copy_((u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()).to(h.dtype))
+    if total is not None:
+        total.copy_(streams.sum(1))
+
+
+def act_rows(x, out, kind, params, gate):
+    """out = act(x) * sigmoid(gate) (gate given).  kind 0: identity; 1: a_p z^2 + z / 2 for z > 0, else
+    a_n (e^z - 1 - z) + z / 2, with params = (a_p, a_n); 2: relu(z)^2."""
+    z = x.float()
+    if kind == 1:
+        ap, an = params.float()[0], params.float()[1]
+        z = torch.where(z > 0, ap * z * z + 0.5 * z, an * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z)
+    elif kind == 2:
+        z = torch.relu(z).pow(2)
+    if gate is not None:
+        z = z * torch.sigmoid(gate.float())
+    out.copy_(z.to(out.dtype))
+
+
+def moe_route(z, correction, topk_idx, topk_w, groups, keep, scale):
+    """Router logits z [M, E] fp32 -> the `top` experts with the largest sigmoid(z) + correction among the experts of
+    the `keep` best of `groups` equal groups of neighbours (a group's score: the sum of its two largest such values);
+    weights: the chosen sigmoid(z) over their sum (+ 1e-20), times scale.  Ties go to the lower index."""
+    M, E = z.shape
+    top = topk_idx.shape[1]
+    s = torch.sigmoid(torch.nan_to_num(z.float(), nan=0.0))
+    choice = s + correction.float()
+    if groups > 1:
+        per = choice.view(M, groups, E // groups)
+        gscore = per.topk(min(2, E // groups), dim=-1).values.sum(-1)
+        order = torch.argsort(gscore, dim=-1, descending=True, stable=True)[:, :keep]
+        allow = torch.zeros(M, groups, dtype=torch.bool).scatter_(1, order, True)
+        choice = per.masked_fill(~allow[:, :, None], float("-inf")).reshape(M, E)
+    idx = torch.argsort(choice, dim=-1, descending=True, stable=True)[:, :top]
+    w = s.gather(1, idx)
+    topk_idx.copy_(idx.to(torch.int32))
+    topk_w.copy_(w / (w.sum(-1, keepdim=True) + 1e-20) * scale)

@@ -38,7 +38,7 @@ struct ScalarNormParams {
 };
 
 struct LatentKvWriteParams {
-  const float* ckr;      // [T, rk + dr] down-projection (latent | shared rotated key part)
+  const float* ckr;      // [T, rk + dr] down-projection (latent | shared rotated key part), rows ld apart
   const void* norm_w;    // [rk]
   const int* positions;  // [T]
   const int* slots;      // [T] cache row (page * kBS + offset), -1 = skip
@@ -47,6 +47,7 @@ struct LatentKvWriteParams {
   int T, rk, dr, rope_len, num_slots;
   float eps;
   int f32;
+  int ld;                // row stride of ckr (a column slice of a wider buffer), rk + dr when contiguous
 };
 
 struct LatentAttnParams {
@@ -87,7 +88,7 @@ struct ConvStateParams {
   int nseq, C, K, rows;  // rows = T
   int f32;
   int ld_in;             // row stride of `in` (a column slice of a wider buffer), C when contiguous
-  int act;               // 0 none, 1 SiLU on the output (the tail keeps the raw inputs)
+  int act;               // 0 none, 1 SiLU on the output (the tail keeps the raw inputs), 2 the row's input added to it
 };
 
 struct LruScanParams {
@@ -140,7 +141,7 @@ struct MoeGroupedParams {
   const void* x;         // [M, W]
   const int* topk_idx;   // [M, top]
   const float* topk_w;   // [M, top]
-  const void* gate;      // [E, F, W]
+  const void* gate;      // [E, F, W], or null: experts without a gate, h = relu(up x)^2
   const void* up;
   const void* down;      // [E, W, F]
   const void* sgate;     // shared expert (slot `top`, expert index E) or null

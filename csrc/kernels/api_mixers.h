@@ -37,7 +37,8 @@ struct NormRopeParams {
   const int* out_rows;   // [T] or null (row t); negative = skip
   void* out_t;           // with out_rows: also into transposed pages [pages, nh, D, kBS] (bf16), token permuted, or null
   int T, nh, D, ldx, ldo, half, rope_len, num_out_rows;
-  int kind;              // 0 none, 1 RMS over the whole row times norm_w, 2 unit vector per head
+  int kind;              // 0 none, 1 RMS over the whole row times norm_w, 2 unit vector per head, 3 RMS per head times
+                         // norm_w [D] (one gain vector for all heads)
   float eps, scale;
   int out_f32;
 };
@@ -103,9 +104,38 @@ struct ScanCarryParams {
   int nseq, H, D, V, decay_kind;
 };
 
+// One pass over the residual streams of every row between two sublayers of a design that carries several of them.
+struct StreamMixParams {
+  float* streams;        // [M, S, W] fp32, rows ld apart
+  const float* y;        // [M * nsum, W] finished sublayer output (a row's nsum parts are summed) or null
+  int nsum;
+  float mult;            // x_t = sum_s mix[s][t] x_s + mult * out_w[t] * y
+  const float* out_w;    // [S] or null (ones)
+  const float* mix;      // [S, S] indexed [from][to], or null (identity)
+  const int* ids;        // [M] token ids (with embed)
+  const void* embed;     // [vocab, W] element type or null: every stream = embed[ids] * embed_scale
+  int vocab;
+  float embed_scale;
+  const float* in_w;     // [S] or null: with h, u = sum_s in_w[s] x_s
+  const float* norm_w;   // [W]
+  void* h;               // [M, W]: u / rms(u) * norm_w (fp32 when h_f32, else the element type), or null
+  float* total;          // [M, W] sum of the streams, or null
+  int M, S, W, ld;
+  float eps;
+  int f32;               // element type of embed (and of h unless h_f32)
+  int h_f32;
+};
+
 }  // namespace dsse
 
 extern "C" {
+hipError_t dsse_stream_mix(const dsse::StreamMixParams* p, hipStream_t st);
+// out [M, F] = act(x) * sigmoid(gate): kind 0 identity, 1 xIELU with params = (a_p, a_n), 2 relu^2; gate may be null
+hipError_t dsse_act_rows(const float* x, int ldx, void* out, int M, int F, int kind, const float* params,
+                         const float* gate, int ldg, int f32, hipStream_t st);
+// group-limited sigmoid routing from fp32 logits [M, E] (E <= 256)
+hipError_t dsse_moe_route(const float* z, const float* corr, int M, int E, int top, int groups, int keep, float scale,
+                          int* topk_idx, float* topk_w, hipStream_t st);
 hipError_t dsse_stream_step(const dsse::StreamStepParams* p, hipStream_t st);
 hipError_t dsse_gated_act(const float* gu, int ldg, void* h, int M, int F, int kind, int f32, hipStream_t st);
 hipError_t dsse_norm_rope_rows(const dsse::NormRopeParams* p, hipStream_t st);

@@ -35,8 +35,8 @@ void i32(const Tensor& t, const char* name) {
   gpu(t, name);
   TORCH_CHECK(t.scalar_type() == at::kInt, name, " must be int32");
 }
-void f32t(const Tensor& t, const char* name) {
-  gpu(t, name);
+void f32t(const Tensor& t, const char* name, bool contiguous = true) {
+  gpu(t, name, contiguous);
   TORCH_CHECK(t.scalar_type() == at::kFloat, name, " must be fp32");
 }
 // element type flag of an activation / weight pair: 1 = fp32, 0 = bf16
@@ -132,15 +132,17 @@ void embed_rows(const Tensor& ids, const Tensor& embed, Tensor& resid, Tensor& x
 
 void latent_kv_write(const Tensor& ckr, const Tensor& norm_w, const Tensor& positions, const Tensor& slots,
                      const Tensor& rope, Tensor& cache, double eps, const OptTensor& vt) {
-  f32t(ckr, "ckr");
+  f32t(ckr, "ckr", false);
   gpu(norm_w, "norm_w");
   i32(positions, "positions");
   i32(slots, "slots");
   f32t(rope, "rope");
   gpu(cache, "cache");
   same(cache, norm_w, "norm_w");
+  TORCH_CHECK(ckr.dim() == 2, "ckr must be [T, rk + dr]");
   const int T = (int)ckr.size(0), D = (int)ckr.size(1), rk = (int)norm_w.numel(), dr = D - rk;
-  TORCH_CHECK(ckr.dim() == 2 && dr >= 0 && dr % 2 == 0, "ckr must be [T, rk + dr], dr even");
+  TORCH_CHECK(dr >= 0 && dr % 2 == 0, "ckr must be [T, rk + dr], dr even");
+  TORCH_CHECK((D == 1 || ckr.stride(1) == 1) && (T <= 1 || ckr.stride(0) >= D), "ckr: unit innermost stride, rows apart");
   TORCH_CHECK(cache.dim() == 3 && cache.size(1) == dsse::kBS && cache.size(2) == D, "cache must be [pages, 32, rk + dr]");
   TORCH_CHECK(rope.dim() == 3 && rope.size(1) == dr / 2 && rope.size(2) == 2, "rope must be [P, dr / 2, 2]");
   TORCH_CHECK(positions.numel() >= T && slots.numel() >= T, "metadata too short");
@@ -152,6 +154,7 @@ void latent_kv_write(const Tensor& ckr, const Tensor& norm_w, const Tensor& posi
   p.rope = reinterpret_cast<const float2*>(rope.data_ptr<float>());
   p.cache = cache.data_ptr();
   p.T = T, p.rk = rk, p.dr = dr, p.rope_len = (int)rope.size(0);
+  p.ld = T > 1 ? (int)ckr.stride(0) : D;
   p.num_slots = (int)(cache.size(0) * dsse::kBS);
   p.eps = (float)eps;
   p.f32 = elem(cache, "cache");
@@ -291,7 +294,7 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, con
   }
   p.C = C, p.K = K, p.rows = (int)in.size(0);
   p.ld_in = (int)in.stride(0);
-  TORCH_CHECK(act == 0 || act == 1, "act: 0 none, 1 SiLU");
+  TORCH_CHECK(act >= 0 && act <= 2, "act: 0 none, 1 SiLU, 2 plus the input");
   p.act = (int)act;
   TORCH_CHECK(p.nseq <= 65535 && (p.rows + 31) / 32 <= 65535, "conv_state: grid too large");
   p.f32 = elem(taps, "taps");
@@ -422,13 +425,12 @@ void moe_ffn(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, cons
 // Grouped form of the routed experts: o [M * S, W] (fp32) = per-(row, slot) expert outputs times their weights, S = top
 // (+ 1 with a shared expert); the caller sums a row's S parts (scalar_norm nsum).  Scratch: sorted [tiles * 64],
 // tile_expert [tiles], num_tiles [1] (int32), h [M * S, ldh] (element type), tiles >= ceil(M S / 64) + experts + 1.
-void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, const Tensor& gate, const Tensor& up,
+void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, const OptTensor& gate, const Tensor& up,
                  const Tensor& down, const OptTensor& sgate, const OptTensor& sup, const OptTensor& sdown, Tensor& sorted,
                  Tensor& tile_expert, Tensor& num_tiles, Tensor& h, Tensor& o) {
   gpu(x, "x");
   i32(topk_idx, "topk_idx");
   f32t(topk_w, "topk_w");
-  gpu(gate, "gate");
   gpu(up, "up");
   gpu(down, "down");
   i32(sorted, "sorted");
@@ -436,14 +438,20 @@ void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, 
   i32(num_tiles, "num_tiles");
   gpu(h, "h");
   f32t(o, "o");
-  same(x, gate, "gate");
   same(x, up, "up");
   same(x, down, "down");
   same(x, h, "h");
   dsse::MoeGroupedParams p{};
   p.M = (int)x.size(0), p.W = (int)x.size(1);
-  TORCH_CHECK(x.dim() == 2 && gate.dim() == 3 && gate.size(2) == p.W && up.sizes() == gate.sizes(), "gate / up must be [E, F, W]");
-  p.E = (int)gate.size(0), p.F = (int)gate.size(1), p.top = (int)topk_idx.size(1);
+  TORCH_CHECK(x.dim() == 2 && up.dim() == 3 && up.size(2) == p.W, "up must be [E, F, W]");
+  if (gate.has_value()) {
+    gpu(*gate, "gate");
+    same(x, *gate, "gate");
+    TORCH_CHECK(gate->sizes() == up.sizes(), "gate must be [E, F, W] like up");
+  } else {
+    TORCH_CHECK(!sgate.has_value(), "experts without a gate have no shared expert");
+  }
+  p.E = (int)up.size(0), p.F = (int)up.size(1), p.top = (int)topk_idx.size(1);
   TORCH_CHECK(down.dim() == 3 && down.size(0) == p.E && down.size(1) == p.W && down.size(2) == p.F, "down must be [E, W, F]");
   TORCH_CHECK(topk_idx.dim() == 2 && topk_idx.size(0) == p.M && topk_w.sizes() == topk_idx.sizes(), "routing shapes");
   p.S = p.top;
@@ -475,7 +483,7 @@ void moe_grouped(const Tensor& x, const Tensor& topk_idx, const Tensor& topk_w, 
   p.x = x.data_ptr();
   p.topk_idx = topk_idx.data_ptr<int>();
   p.topk_w = topk_w.data_ptr<float>();
-  p.gate = gate.data_ptr();
+  p.gate = gate.has_value() ? gate->data_ptr() : nullptr;
   p.up = up.data_ptr();
   p.down = down.data_ptr();
   p.sorted = sorted.data_ptr<int>();
@@ -508,7 +516,7 @@ void moe_topk(const Tensor& logits, Tensor& topk_idx, Tensor& topk_w) {
 TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("gemm_rm(Tensor x, Tensor w, Tensor(a!) out, Tensor? bias=None, int act=0) -> ()");
   m.def("scalar_norm(Tensor? y, Tensor g, Tensor(a!) resid, Tensor(b!) xb, float eps, int nsum=1) -> ()");
-  m.def("moe_grouped(Tensor x, Tensor topk_idx, Tensor topk_w, Tensor gate, Tensor up, Tensor down, Tensor? sgate, "
+  m.def("moe_grouped(Tensor x, Tensor topk_idx, Tensor topk_w, Tensor? gate, Tensor up, Tensor down, Tensor? sgate, "
         "Tensor? sup, Tensor? sdown, Tensor(a!) sorted, Tensor(b!) tile_expert, Tensor(c!) num_tiles, Tensor(d!) h, "
         "Tensor(e!) o) -> ()");
   m.def("embed_rows(Tensor ids, Tensor embed, Tensor(a!) resid, Tensor(b!) xb) -> ()");

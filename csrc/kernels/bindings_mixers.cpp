@@ -128,10 +128,10 @@ void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& posi
   p.T = (int)x.size(0), p.nh = (int)x.size(1), p.D = (int)x.size(2);
   p.ldx = (int)x.stride(0);
   p.x = x.data_ptr<float>();
-  TORCH_CHECK(kind >= 0 && kind <= 2 && p.D <= 512, "kind 0..2, head width <= 512");
+  TORCH_CHECK(kind >= 0 && kind <= 3 && p.D <= 512, "kind 0..3, head width <= 512");
   p.kind = (int)kind;
-  p.norm_w = opt_f32(norm_w, "norm_w", (int64_t)p.nh * p.D);
-  TORCH_CHECK(kind != 1 || p.norm_w, "kind 1 needs norm_w");
+  p.norm_w = opt_f32(norm_w, "norm_w", kind == 3 ? (int64_t)p.D : (int64_t)p.nh * p.D);
+  TORCH_CHECK((kind != 1 && kind != 3) || p.norm_w, "kinds 1 and 3 need norm_w");
   if (rope.has_value() && rope->numel() > 0) {
     f32t(*rope, "rope");
     i32(positions, "positions");
@@ -429,7 +429,105 @@ void logit_cap(Tensor& logits, double scale, double cap) {
 
 }  // namespace
 
+void stream_mix(const OptTensor& y, int64_t nsum, double mult, Tensor& streams, const OptTensor& ids,
+                const OptTensor& embed, double embed_scale, const OptTensor& out_w, const OptTensor& mix,
+                const OptTensor& in_w, const OptTensor& norm_w, double eps, const OptTensor& h, const OptTensor& total) {
+  f32t(streams, "streams", false);
+  TORCH_CHECK(streams.dim() == 3, "streams must be [M, S, W]");
+  dsse::StreamMixParams p{};
+  p.M = (int)streams.size(0), p.S = (int)streams.size(1), p.W = (int)streams.size(2);
+  TORCH_CHECK(p.S >= 1 && p.S <= 8, "1..8 streams");
+  TORCH_CHECK((p.W == 1 || streams.stride(2) == 1) && (p.S == 1 || streams.stride(1) == p.W) &&
+                  (p.M <= 1 || streams.stride(0) >= (int64_t)p.S * p.W),
+              "streams: adjacent copies of contiguous rows");
+  p.ld = p.M > 1 ? (int)streams.stride(0) : p.S * p.W;
+  p.streams = streams.data_ptr<float>();
+  p.nsum = (int)nsum, p.mult = (float)mult, p.embed_scale = (float)embed_scale, p.eps = (float)eps;
+  TORCH_CHECK(nsum >= 1, "nsum >= 1");
+  p.f32 = 1;
+  bool typed = false;
+  if (y.has_value()) {
+    f32t(*y, "y");
+    TORCH_CHECK(y->dim() == 2 && y->size(0) == (int64_t)p.M * nsum && y->size(1) == p.W, "y must be [M * nsum, W]");
+    p.y = y->data_ptr<float>();
+    p.out_w = opt_f32(out_w, "out_w", p.S);
+    p.mix = opt_f32(mix, "mix", (int64_t)p.S * p.S);
+  }
+  if (embed.has_value()) {
+    TORCH_CHECK(ids.has_value(), "embed needs ids");
+    i32(*ids, "ids");
+    gpu(*embed, "embed");
+    TORCH_CHECK(embed->dim() == 2 && embed->size(1) == p.W && ids->numel() >= p.M, "embed must be [vocab, W]");
+    p.ids = ids->data_ptr<int>();
+    p.embed = embed->data_ptr();
+    p.vocab = (int)embed->size(0);
+    p.f32 = elem(*embed, "embed");
+    typed = true;
+  }
+  if (h.has_value()) {
+    TORCH_CHECK(in_w.has_value() && norm_w.has_value(), "h needs in_w and norm_w");
+    p.in_w = opt_f32(in_w, "in_w", p.S);
+    p.norm_w = opt_f32(norm_w, "norm_w", p.W);
+    gpu(*h, "h");
+    TORCH_CHECK(h->dim() == 2 && h->size(0) == p.M && h->size(1) == p.W, "h must be [M, W]");
+    const int f = elem(*h, "h");
+    if (f) {
+      p.h_f32 = 1;  // an fp32 h beside a bf16 embedding is the mixed kernel
+    } else {
+      TORCH_CHECK(!typed || p.f32 == 0, "a bf16 h needs a bf16 embedding");
+      p.f32 = 0;
+    }
+    p.h = h->data_ptr();
+  }
+  if (total.has_value()) {
+    f32t(*total, "total");
+    TORCH_CHECK(total->dim() == 2 && total->size(0) == p.M && total->size(1) == p.W, "total must be [M, W]");
+    p.total = total->data_ptr<float>();
+  }
+  DSSE_CHECK_HIP(dsse_stream_mix(&p, cur_stream()));
+}
+
+void act_rows(const Tensor& x, Tensor& out, int64_t kind, const OptTensor& params, const OptTensor& gate) {
+  col_view(x, "x");
+  gpu(out, "out");
+  TORCH_CHECK(out.dim() == 2 && out.sizes() == x.sizes(), "out must be [M, F] like x");
+  TORCH_CHECK(kind >= 0 && kind <= 2, "kind: 0 identity, 1 xIELU, 2 relu^2");
+  const float* pp = opt_f32(params, "params", 2);
+  TORCH_CHECK(kind != 1 || pp, "xIELU needs its two constants");
+  const float* g = nullptr;
+  int ldg = 0;
+  if (gate.has_value()) {
+    col_view(*gate, "gate");
+    TORCH_CHECK(gate->sizes() == x.sizes(), "gate must be [M, F] like x");
+    g = gate->data_ptr<float>();
+    ldg = (int)gate->stride(0);
+  }
+  DSSE_CHECK_HIP(dsse_act_rows(x.data_ptr<float>(), (int)x.stride(0), out.data_ptr(), (int)x.size(0), (int)x.size(1),
+                               (int)kind, pp, g, ldg, elem(out, "out"), cur_stream()));
+}
+
+void moe_route(const Tensor& z, const Tensor& correction, Tensor& topk_idx, Tensor& topk_w, int64_t groups, int64_t keep,
+               double scale) {
+  f32t(z, "z");
+  f32t(correction, "correction");
+  i32(topk_idx, "topk_idx");
+  f32t(topk_w, "topk_w");
+  TORCH_CHECK(z.dim() == 2 && topk_idx.dim() == 2, "z must be [M, E], topk_idx [M, top]");
+  const int M = (int)z.size(0), E = (int)z.size(1), top = (int)topk_idx.size(1);
+  TORCH_CHECK(topk_idx.size(0) == M && topk_w.sizes() == topk_idx.sizes() && correction.numel() == E, "routing shapes");
+  TORCH_CHECK(E >= 1 && E <= 256 && groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 &&
+                  top <= keep * (E / groups),
+              "routing: E <= 256, equal groups, 1 <= keep <= groups, top <= experts of the kept groups");
+  DSSE_CHECK_HIP(dsse_moe_route(z.data_ptr<float>(), correction.data_ptr<float>(), M, E, top, (int)groups, (int)keep,
+                                (float)scale, topk_idx.data_ptr<int>(), topk_w.data_ptr<float>(), cur_stream()));
+}
+
 TORCH_LIBRARY_FRAGMENT(dsse, m) {
+  m.def("stream_mix(Tensor? y, int nsum, float mult, Tensor(a!) streams, Tensor? ids, Tensor? embed, float embed_scale, "
+        "Tensor? out_w, Tensor? mix, Tensor? in_w, Tensor? norm_w, float eps, Tensor(b!)? h, Tensor(c!)? total) -> ()");
+  m.def("act_rows(Tensor x, Tensor(a!) out, int kind, Tensor? params=None, Tensor? gate=None) -> ()");
+  m.def("moe_route(Tensor z, Tensor correction, Tensor(a!) topk_idx, Tensor(b!) topk_w, int groups, int keep, "
+        "float scale) -> ()");
   m.def("stream_step(Tensor? y, float mult, Tensor(a!) resid, Tensor? ids, Tensor? embed, Tensor? vec, Tensor? alpha, "
         "Tensor? w, Tensor? b, Tensor(b!)? xb) -> ()");
   m.def("gated_act(Tensor gu, Tensor(a!) h, int kind=1) -> ()");
@@ -450,6 +548,9 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
 }
 
 TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
+  m.impl("stream_mix", &stream_mix);
+  m.impl("act_rows", &act_rows);
+  m.impl("moe_route", &moe_route);
   m.impl("stream_step", &stream_step);
   m.impl("gated_act", &gated_act);
   m.impl("norm_rope_rows", &norm_rope_rows);

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(LatentKvWriteParam
   const int slot = p.slots[row];
   if (slot < 0 || slot >= p.num_slots) return;  // uniform per workgroup
   const int D = p.rk + p.dr;
-  const float* src = p.ckr + (int64_t)row * D;
+  const float* src = p.ckr + (int64_t)row * p.ld;
   T* dst = reinterpret_cast<T*>(p.cache) + (int64_t)slot * D;
   float ss = 0.f;
   for (int d = threadIdx.x; d < p.rk; d += blockDim.x) ss += src[d] * src[d];

@@ -224,8 +224,11 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
   const int Fe = sh ? p.Fs : p.F;
   if ((int)blockIdx.x * 16 >= Fe) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
-  const T* gate = sh ? reinterpret_cast<const T*>(p.sgate) : reinterpret_cast<const T*>(p.gate) + (int64_t)e * p.F * p.W;
+  const bool gated = p.gate != nullptr;  // uniform: experts without a gate are down(relu(up x)^2)
   const T* up = sh ? reinterpret_cast<const T*>(p.sup) : reinterpret_cast<const T*>(p.up) + (int64_t)e * p.F * p.W;
+  const T* gate = !gated ? up
+                         : (sh ? reinterpret_cast<const T*>(p.sgate)
+                               : reinterpret_cast<const T*>(p.gate) + (int64_t)e * p.F * p.W);
   const int* ids = p.sorted + t * kMoeRows;
   // an expert's ids fill its tiles from the front: a 16-row sub-tile is empty when its first id is a pad
   const T* xr[4];
@@ -247,24 +250,26 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGroupedParams p) {
   for (int i = 0; i < 4; ++i) ag[i] = au[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = wave * F::KS; k0 < p.W; k0 += 4 * F::KS) {
     const int k = k0 + F::PER * g;
-    const typename F::V bg = load_frag<T>(gr, k, p.W, fv, vec), bu = load_frag<T>(ur, k, p.W, fv, vec);
+    const typename F::V bu = load_frag<T>(ur, k, p.W, fv, vec);
+    const typename F::V bg = gated ? load_frag<T>(gr, k, p.W, fv, vec) : bu;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (!live[i]) continue;  // uniform over the workgroup
       const typename F::V a = load_frag<T>(xr[i], k, p.W, xv[i], vec);
-      ag[i] = mma(a, bg, ag[i]);
+      if (gated) ag[i] = mma(a, bg, ag[i]);
       au[i] = mma(a, bu, au[i]);
     }
   }
-  reduce4(ag, red, wave, lane);
+  if (gated) reduce4(ag, red, wave, lane);
   reduce4(au, red, wave, lane);
   if (!fv || !live[wave]) return;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int id2 = ids[16 * wave + 4 * g + j];
     if (id2 < 0) continue;
-    const float gv = ag[0][j];
-    reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] = (T)(gv / (1.0f + expf(-gv)) * au[0][j]);
+    const float gv = ag[0][j], uv = au[0][j];
+    reinterpret_cast<T*>(p.h)[(int64_t)id2 * p.ldh + f] =
+        (T)(gated ? gv / (1.0f + expf(-gv)) * uv : (uv > 0.0f ? uv * uv : 0.0f));
   }
 }
 
@@ -336,16 +341,18 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(MoeGroupedParams p) {
   const int e = p.tile_expert[t];
   const bool sh = e >= p.E;
   const int Fe = sh ? p.Fs : p.F;
-  const int K = MODE == 0 ? p.W : Fe;          // reduction length
-  const int N = MODE == 0 ? Fe : p.W;          // weight rows of one kind
+  const int K = MODE == 1 ? Fe : p.W;          // reduction length
+  const int N = MODE == 1 ? p.W : Fe;          // weight rows of one kind
   const int n0 = blockIdx.x * (MODE == 0 ? 64 : 128);
   if (n0 >= N) return;
   const int* ids = p.sorted + t * kMoeRows;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
-  const bf16* X = reinterpret_cast<const bf16*>(MODE == 0 ? p.x : p.h);
-  const int ldx = MODE == 0 ? p.W : p.ldh;
-  const bf16 *w0, *w1;  // MODE 0: gate, up; MODE 1: down (w1 unused)
-  if (MODE == 0) {
+  const bf16* X = reinterpret_cast<const bf16*>(MODE == 1 ? p.h : p.x);
+  const int ldx = MODE == 1 ? p.ldh : p.W;
+  const bf16 *w0, *w1;  // MODE 0: gate, up; MODE 1: down (w1 unused); MODE 2: up alone (experts without a gate)
+  if (MODE == 2) {
+    w0 = w1 = reinterpret_cast<const bf16*>(p.up) + (int64_t)e * p.F * p.W;
+  } else if (MODE == 0) {
     w0 = sh ? reinterpret_cast<const bf16*>(p.sgate) : reinterpret_cast<const bf16*>(p.gate) + (int64_t)e * p.F * p.W;
     w1 = sh ? reinterpret_cast<const bf16*>(p.sup) : reinterpret_cast<const bf16*>(p.up) + (int64_t)e * p.F * p.W;
   } else {
@@ -360,7 +367,7 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(MoeGroupedParams p) {
   for (int i = 0; i < 2; ++i) {
     const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
     const int id = ids[row];
-    ap[i] = id >= 0 ? X + (int64_t)(MODE == 0 ? id / p.S : id) * ldx : nullptr;
+    ap[i] = id >= 0 ? X + (int64_t)(MODE == 1 ? id : id / p.S) * ldx : nullptr;
     ak[i] = 8 * pc;
     ao[i] = row * kLdsRow + 8 * pc;
   }
@@ -433,6 +440,13 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(MoeGroupedParams p) {
         if (f >= N) continue;
         const float gv = acc[i][0][j];
         reinterpret_cast<bf16*>(p.h)[(int64_t)id * p.ldh + f] = (bf16)(gv / (1.0f + expf(-gv)) * acc[i][1][j]);
+      } else if (MODE == 2) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int f = n0 + 32 * wave + 16 * q + r;
+          const float uv = acc[i][q][j];
+          if (f < N) reinterpret_cast<bf16*>(p.h)[(int64_t)id * p.ldh + f] = (bf16)(uv > 0.0f ? uv * uv : 0.0f);
+        }
       } else {
         const int row = id / p.S, k = id % p.S;
         const float wgt = k < p.top ? p.topk_w[row * p.top + k] : 1.0f;
@@ -474,8 +488,9 @@ extern "C" hipError_t dsse_moe_grouped(const dsse::MoeGroupedParams* p, hipStrea
   dim3 g1((fmax + 15) / 16, p->max_tiles), g2((p->W + 15) / 16, p->max_tiles);
   // prompt-sized steps in bf16 with 16-byte-aligned rows: operands staged through LDS
   if (!p->f32 && p->lds_tiles && p->W % 8 == 0 && p->F % 8 == 0 && p->Fs % 8 == 0 && p->ldh % 8 == 0) {
-    dim3 l1((fmax + 63) / 64, p->max_tiles), l2((p->W + 127) / 128, p->max_tiles);
-    hipLaunchKernelGGL(dsse::moe_tile_lds_kernel<0>, l1, dim3(256), 0, st, *p);
+    dim3 l1((fmax + 63) / 64, p->max_tiles), l2((p->W + 127) / 128, p->max_tiles), l3((fmax + 127) / 128, p->max_tiles);
+    if (p->gate) hipLaunchKernelGGL(dsse::moe_tile_lds_kernel<0>, l1, dim3(256), 0, st, *p);
+    else hipLaunchKernelGGL(dsse::moe_tile_lds_kernel<2>, l3, dim3(256), 0, st, *p);
     hipLaunchKernelGGL(dsse::moe_tile_lds_kernel<1>, l2, dim3(256), 0, st, *p);
     return hipGetLastError();
   }

@@ -3,7 +3,8 @@
 //
 //   conv_state   out[t, c] = b[c] + sum_k taps[c, k] * in[t - (K - 1) + k, c]; inputs before the step's first row come
 //                from the slot's tail (the last K - 1 inputs of the sequence), an empty (zero) history at position 0.  The
-//                tail is rewritten with the step's last K - 1 inputs (shifted in place when the step is shorter).
+//                tail is rewritten with the step's last K - 1 inputs (shifted in place when the step is shorter).  An
+//                optional SiLU on the output, or the row's own input added to it (in + conv(in)).
 //   lru_scan     r = sigmoid(gate_r), i = sigmoid(gate_i), log a = -c r softplus(lam), S = a S + sqrt(1 - a^2) i u,
 //                out = S * y.  The state S is fp32 and lives in the sequence's slot; a sequence's first step starts from
 //                S = 0 (position 0 is not special-cased beyond that: the recurrence's own formula applies to it).
@@ -48,6 +49,7 @@ __global__ __launch_bounds__(256) void conv_state_kernel(ConvStateParams p) {
       v += (float)taps[k] * x;
     }
     if (p.act == 1) v = v / (1.0f + expf(-v));
+    else if (p.act == 2) v += in[(int64_t)t * p.ld_in] + ib;
     p.out[(int64_t)(row0 + t) * p.C + c] = v;
     if (p.out_b) reinterpret_cast<T*>(p.out_b)[(int64_t)(row0 + t) * p.C + c] = (T)v;
   }

@@ -3,7 +3,8 @@
 //   stream_step      resid += mult * y + embed[id] + vec, then xb = tanh(alpha * resid) * w + b (the element-wise norm
 //                    that needs no row statistic, so the add and the norm are one pass over the row)
 //   gated_act        h = act(gate) * up from the fused gate | up projection's fp32 output (SiLU or tanh-form gelu)
-//   norm_rope_rows   a row of heads: RMS norm over the whole row with a gain, or a unit vector per head, or nothing;
+//   norm_rope_rows   a row of heads: RMS norm over the whole row with a gain, a unit vector per head, an RMS norm per
+//                    head with one gain vector for all heads, or nothing;
 //                    rotate-half rotation of each head's leading coordinates; a scale; written to a chosen output row
 //                    (a cache row: keys and values go straight into their pages) in fp32 or bf16
 //   gate_math        decays and gates in place: exp(-exp(A) softplus(x + dt)), sigmoid(x), sigmoid(x)^(1/tau)
@@ -101,13 +102,15 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(NormRopeParams p) {
     const bool on = h < p.nh;
     const float* xh = x + (on ? h : 0) * p.D;
     float inv = inv_row;
-    if (p.kind == 2) {
+    if (p.kind >= 2) {
       float ss = 0.f;
       for (int i = lane; i < p.D; i += 64) ss += xh[i] * xh[i];
-      inv = 1.0f / sqrtf(wave_sum(ss) + p.eps);
+      ss = wave_sum(ss);
+      inv = 1.0f / sqrtf((p.kind == 3 ? ss / (float)p.D : ss) + p.eps);
     }
     if (on)
-      for (int i = lane; i < p.D; i += 64) s[i] = xh[i] * inv * (p.kind == 1 ? p.norm_w[h * p.D + i] : 1.0f);
+      for (int i = lane; i < p.D; i += 64)
+        s[i] = xh[i] * inv * (p.kind == 1 ? p.norm_w[h * p.D + i] : (p.kind == 3 ? p.norm_w[i] : 1.0f));
     __syncthreads();  // the strip is written before it is read
     if (on)
       for (int i = lane; i < p.D; i += 64) {

@@ -602,7 +602,9 @@ class LayeredRunner(RunnerBase):
         o = d["o"][:M * H * dv].view(M, H, dv)
         ao = d["ao"][:M * H * dv].view(M, H * dv)
         self._lin(d["xb"], Lw.big, Lw.big_t, big)
-        ops.norm_rope_rows(big[:, :qr].unsqueeze(1), Lw.dq_norm, pos, None, cq.unsqueeze(1), None, 1, self.cfg.eps, 1.0)
+        # the query latent's RMS norm: one "stream" with weight 1 (any width, read in place from the fused output)
+        ops.stream_mix(None, 1, 0.0, big[:, :qr].unsqueeze(1), in_w=self.w.ones[:1], norm_w=Lw.dq_norm, eps=self.cfg.eps,
+                       h=cq)
         self._lin(cq, Lw.uq, Lw.uq_t, q.view(M, H * (dn + dr)))
         ops.latent_kv_write(big[:, qr:qr + rk + dr], Lw.dkv_norm, pos, slots, rope, cache, self.cfg.eps, vt)
         ops.gemm_rm(q[:, :, :dn].permute(1, 0, 2), Lw.uk_t, qabs.permute(1, 0, 2))

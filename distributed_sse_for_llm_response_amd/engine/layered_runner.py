@@ -607,7 +607,10 @@ class LayeredRunner(RunnerBase):
                        h=cq)
         self._lin(cq, Lw.uq, Lw.uq_t, q.view(M, H * (dn + dr)))
         ops.latent_kv_write(big[:, qr:qr + rk + dr], Lw.dkv_norm, pos, slots, rope, cache, self.cfg.eps, vt)
-        ops.gemm_rm(q[:, :, :dn].permute(1, 0, 2), Lw.uk_t, qabs.permute(1, 0, 2))
+        if dn > 0:
+            ops.gemm_rm(q[:, :, :dn].permute(1, 0, 2), Lw.uk_t, qabs.permute(1, 0, 2))
+        else:  # heads without an unrotated part: nothing folds into the latent
+            qabs.zero_()
         for g in groups:
             if vt is not None:
                 if g["qt"] == 1:

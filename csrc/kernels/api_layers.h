@@ -83,12 +83,13 @@ struct ConvStateParams {
   const int* q_len;
   const int* ctx_len;
   const int* state_slot;
-  float* out;            // [T, C] fp32
+  float* out;            // [T, C] fp32 or null
   void* out_b;           // [T, C] element type (the gates' GEMM input) or null
   int nseq, C, K, rows;  // rows = T
   int f32;
   int ld_in;             // row stride of `in` (a column slice of a wider buffer), C when contiguous
   int act;               // 0 none, 1 SiLU on the output (the tail keeps the raw inputs), 2 the row's input added to it
+  int single;            // 1: every sequence has few rows (a decode step: one): the convolution kernel also moves the tail
 };
 
 struct LruScanParams {

@@ -248,19 +248,23 @@ void seq_meta(const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len,
 }
 
 void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, const OptTensor& tail, const Tensor& q_start,
-                const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, Tensor& out, const OptTensor& out_b,
-                const OptTensor& in_bias, int64_t act) {
+                const Tensor& q_len, const Tensor& ctx_len, const Tensor& state_slot, const OptTensor& out,
+                const OptTensor& out_b, const OptTensor& in_bias, int64_t act, bool single) {
   gpu(in, "in", false);
   TORCH_CHECK(in.scalar_type() == at::kFloat, "in must be fp32");
   gpu(taps, "taps");
-  f32t(out, "out");
   dsse::ConvStateParams p{};
   seq_meta(q_start, q_len, ctx_len, state_slot, p.nseq);
   TORCH_CHECK(in.dim() == 2 && taps.dim() == 2, "in must be [T, C], taps [C, K]");
   const int C = (int)in.size(1), K = (int)taps.size(1);
   TORCH_CHECK(taps.size(0) == C && K >= 1, "taps must be [C, K]");
   TORCH_CHECK(C == 1 || in.stride(1) == 1, "in needs a unit innermost stride");
-  TORCH_CHECK(out.sizes() == in.sizes(), "out must match in");
+  if (out.has_value()) {
+    f32t(*out, "out");
+    TORCH_CHECK(out->sizes() == in.sizes(), "out must match in");
+    p.out = out->data_ptr<float>();
+  }
+  TORCH_CHECK(out.has_value() || out_b.has_value(), "conv_state needs out or out_b");
   if (out_b.has_value()) {
     gpu(*out_b, "out_b");
     same(taps, *out_b, "out_b");
@@ -285,7 +289,7 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, con
   p.q_len = q_len.data_ptr<int>();
   p.ctx_len = ctx_len.data_ptr<int>();
   p.state_slot = state_slot.data_ptr<int>();
-  p.out = out.data_ptr<float>();
+  p.single = single ? 1 : 0;
   if (in_bias.has_value()) {
     gpu(*in_bias, "in_bias");
     same(taps, *in_bias, "in_bias");
@@ -296,7 +300,7 @@ void conv_state(const Tensor& in, const Tensor& taps, const OptTensor& bias, con
   p.ld_in = (int)in.stride(0);
   TORCH_CHECK(act >= 0 && act <= 2, "act: 0 none, 1 SiLU, 2 plus the input");
   p.act = (int)act;
-  TORCH_CHECK(p.nseq <= 65535 && (p.rows + 31) / 32 <= 65535, "conv_state: grid too large");
+  TORCH_CHECK(p.nseq <= 65535 && (p.rows + 7) / 8 <= 65535, "conv_state: grid too large");
   p.f32 = elem(taps, "taps");
   DSSE_CHECK_HIP(dsse_conv_state(&p, cur_stream()));
 }
@@ -526,7 +530,8 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor rope, Tensor(a!) out, int window, float scale, "
         "int qt, Tensor? vt=None, int hp=1, Tensor(b!)? part=None, int nparts=1) -> ()");
   m.def("conv_state(Tensor inp, Tensor taps, Tensor? bias, Tensor(a!)? tail, Tensor q_start, Tensor q_len, "
-        "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, Tensor(c!)? out_b, Tensor? in_bias=None, int act=0) -> ()");
+        "Tensor ctx_len, Tensor state_slot, Tensor(b!)? out, Tensor(c!)? out_b, Tensor? in_bias=None, int act=0, "
+        "bool single=False) -> ()");
   m.def("lru_scan(Tensor u, Tensor(c!) gates, Tensor y, Tensor lam, Tensor(a!) state, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float c, Tensor? y_bias=None, bool coeff=True, "
         "Tensor(d!)? scratch=None) -> ()");

@@ -30,19 +30,50 @@ DEV float block_sum(float v, float* red) {
   return s;
 }
 
-// One workgroup per row.  The mixed streams go back to memory in the first sweep; the norm's second sweep re-forms u
-// from them (the row's S * W floats are still in the nearest cache), so no width limit comes from LDS or registers.
-template <typename T, typename HT>
+// One workgroup per row, the stream count a template parameter (every per-stream array is indexed statically and lives
+// in registers).  A thread owns groups of VEC consecutive channels (VEC = 4 when the width allows 16-byte accesses):
+// it reads the S old values of each, mixes, writes the S new ones, and keeps u = sum_s in[s] x_s of up to kKeep groups
+// in registers for the norm's second sweep; wider rows re-form the rest from the streams it has just written (the same
+// thread wrote those addresses).
+constexpr int kKeep = 4;
+
+template <int VEC>
+struct Pack { float v[VEC]; };
+
+template <int VEC>
+DEV Pack<VEC> ld_pack(const float* p) {
+  Pack<VEC> r;
+  if (VEC == 4) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    r.v[0] = t[0], r.v[1] = t[1], r.v[2] = t[2], r.v[3] = t[3];
+  } else {
+    r.v[0] = p[0];
+  }
+  return r;
+}
+template <int VEC>
+DEV void st_pack(float* p, const Pack<VEC>& r) {
+  if (VEC == 4) *reinterpret_cast<f32x4*>(p) = f32x4{r.v[0], r.v[1], r.v[2], r.v[3]};
+  else p[0] = r.v[0];
+}
+template <int VEC, typename T>
+DEV void st_elem(T* p, const Pack<VEC>& r) {
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) p[j] = (T)r.v[j];
+}
+
+template <typename T, typename HT, int S, int VEC>
 __global__ __launch_bounds__(256) void stream_mix_kernel(StreamMixParams p) {
   __shared__ float red[4];
-  __shared__ float s_mix[kMaxStreams * kMaxStreams], s_in[kMaxStreams], s_out[kMaxStreams];
-  const int row = blockIdx.x, S = p.S, W = p.W;
-  for (int i = threadIdx.x; i < S * S; i += blockDim.x) s_mix[i] = p.mix ? p.mix[i] : (i / S == i % S ? 1.0f : 0.0f);
-  for (int i = threadIdx.x; i < S; i += blockDim.x) {
-    s_in[i] = p.in_w ? p.in_w[i] : 0.0f;
-    s_out[i] = p.y ? p.mult * (p.out_w ? p.out_w[i] : 1.0f) : 0.0f;
+  const int row = blockIdx.x, W = p.W;
+  float m_mix[S][S], m_in[S], m_out[S];
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    m_in[s] = p.in_w ? p.in_w[s] : 0.0f;
+    m_out[s] = p.y ? p.mult * (p.out_w ? p.out_w[s] : 1.0f) : 0.0f;
+#pragma unroll
+    for (int t = 0; t < S; ++t) m_mix[s][t] = p.mix ? p.mix[s * S + t] : (s == t ? 1.0f : 0.0f);
   }
-  __syncthreads();
   float* x = p.streams + (int64_t)row * p.ld;
   const T* e = nullptr;
   if (p.embed) {
@@ -53,54 +84,84 @@ __global__ __launch_bounds__(256) void stream_mix_kernel(StreamMixParams p) {
   const float* y = p.y ? p.y + (int64_t)row * p.nsum * W : nullptr;
   float* tot = p.total ? p.total + (int64_t)row * W : nullptr;
   const bool rewrite = e || y;
+  Pack<VEC> keep[kKeep];
   float ss = 0.f;
-  for (int d = threadIdx.x; d < W; d += blockDim.x) {
-    float xs[kMaxStreams], xn[kMaxStreams];
+  int it = 0;
+  for (int d = threadIdx.x * VEC; d < W; d += 256 * VEC, ++it) {
+    Pack<VEC> xs[S], xn[S];
     if (e) {
-      const float v = (float)e[d] * p.embed_scale;
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s) xs[s] = v;
-    } else {
+      for (int j = 0; j < VEC; ++j) {
+        const float v = (float)e[d + j] * p.embed_scale;
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s) xs[s] = s < S ? x[(int64_t)s * W + d] : 0.0f;
-    }
-    if (y) {
-      float yv = 0.f;
-      for (int k = 0; k < p.nsum; ++k) yv += y[(int64_t)k * W + d];
-#pragma unroll
-      for (int t = 0; t < kMaxStreams; ++t) {
-        if (t >= S) break;
-        float v = s_out[t] * yv;
-#pragma unroll
-        for (int s = 0; s < kMaxStreams; ++s)
-          if (s < S) v += s_mix[s * S + t] * xs[s];
-        xn[t] = v;
+        for (int s = 0; s < S; ++s) xs[s].v[j] = v;
       }
     } else {
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s) xn[s] = xs[s];
+      for (int s = 0; s < S; ++s) xs[s] = ld_pack<VEC>(x + (int64_t)s * W + d);
     }
-    float u = 0.f, sum = 0.f;
+    if (y) {
+      Pack<VEC> yv = ld_pack<VEC>(y + d);
+      for (int k = 1; k < p.nsum; ++k) {
+        const Pack<VEC> t = ld_pack<VEC>(y + (int64_t)k * W + d);
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s) {
-      if (s >= S) break;
-      if (rewrite) x[(int64_t)s * W + d] = xn[s];
-      u += s_in[s] * xn[s];
-      sum += xn[s];
+        for (int j = 0; j < VEC; ++j) yv.v[j] += t.v[j];
+      }
+#pragma unroll
+      for (int t = 0; t < S; ++t)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          float v = m_out[t] * yv.v[j];
+#pragma unroll
+          for (int s = 0; s < S; ++s) v += m_mix[s][t] * xs[s].v[j];
+          xn[t].v[j] = v;
+        }
+    } else {
+#pragma unroll
+      for (int s = 0; s < S; ++s) xn[s] = xs[s];
     }
-    ss += u * u;
-    if (tot) tot[d] = sum;
+    Pack<VEC> u, sum;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float uu = 0.f, sm = 0.f;
+#pragma unroll
+      for (int s = 0; s < S; ++s) uu += m_in[s] * xn[s].v[j], sm += xn[s].v[j];
+      u.v[j] = uu, sum.v[j] = sm;
+      ss += uu * uu;
+    }
+    if (rewrite)
+#pragma unroll
+      for (int s = 0; s < S; ++s) st_pack<VEC>(x + (int64_t)s * W + d, xn[s]);
+    if (tot) st_pack<VEC>(tot + d, sum);
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k)
+      if (k == it) keep[k] = u;
   }
   if (!p.h) return;  // uniform
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)W + p.eps);
   HT* h = reinterpret_cast<HT*>(p.h) + (int64_t)row * W;
-  for (int d = threadIdx.x; d < W; d += blockDim.x) {  // the same thread wrote these addresses in the first sweep
-    float u = 0.f;
+  it = 0;
+  for (int d = threadIdx.x * VEC; d < W; d += 256 * VEC, ++it) {
+    Pack<VEC> u;
+    if (it < kKeep) {
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
-      if (s < S) u += s_in[s] * x[(int64_t)s * W + d];
-    h[d] = (HT)(u * inv * p.norm_w[d]);
+      for (int k = 0; k < kKeep; ++k)
+        if (k == it) u = keep[k];
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) u.v[j] = 0.f;
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+        const Pack<VEC> t = ld_pack<VEC>(x + (int64_t)s * W + d);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) u.v[j] += m_in[s] * t.v[j];
+      }
+    }
+    const Pack<VEC> g = ld_pack<VEC>(p.norm_w + d);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) u.v[j] *= inv * g.v[j];
+    st_elem<VEC, HT>(h + d, u);
   }
 }
 
@@ -123,28 +184,28 @@ __global__ __launch_bounds__(256) void act_rows_kernel(const float* x, int ldx, 
   }
 }
 
-// One thread per row; E <= kMaxRouteExperts choice scores live in the thread's scratch.  Ties go to the lower index.
+// One wave per row, E <= kMaxRouteExperts.  Choice scores sit in LDS; lanes own groups for the group scores and
+// ranks, and every pick is a wave-wide argmax (ties go to the lower index, as in the reference).
 constexpr int kMaxRouteExperts = 256;
 
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr, int M,
                                                        int E, int top, int groups, int keep, float scale, int* topk_idx,
                                                        float* topk_w) {
-  const int row = blockIdx.x * blockDim.x + threadIdx.x;
-  if (row >= M) return;
+  __shared__ float choice[kMaxRouteExperts], score[kMaxRouteExperts], gs[kMaxRouteExperts];
+  const int row = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (int64_t)row * E;
-  int* idx = topk_idx + (int64_t)row * top;
-  float* wt = topk_w + (int64_t)row * top;
-  float choice[kMaxRouteExperts];
   const float ninf = -__builtin_inff();
-  for (int e = 0; e < E; ++e) {
+  for (int e = lane; e < E; e += 64) {
     float v = zr[e];
     v = v == v ? v : 0.0f;
-    choice[e] = 1.0f / (1.0f + expf(-v)) + corr[e];
+    const float sg = 1.0f / (1.0f + expf(-v));
+    score[e] = sg;
+    choice[e] = sg + corr[e];
   }
+  __syncthreads();
   if (groups > 1) {
     const int per = E / groups;
-    float gs[kMaxRouteExperts];  // a group's score: the sum of its two largest choice scores
-    for (int o = 0; o < groups; ++o) {
+    for (int o = lane; o < groups; o += 64) {  // a group's score: the sum of its two largest choice scores
       float a = ninf, b = ninf;
       for (int j = 0; j < per; ++j) {
         const float c = choice[o * per + j];
@@ -153,34 +214,45 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
       }
       gs[o] = per > 1 ? a + b : a;
     }
+    __syncthreads();
     // rank of a group = groups with a larger score (or the same score and a lower index); eligible when rank < keep
-    for (int g = 0; g < groups; ++g) {
+    for (int g = lane; g < groups; g += 64) {
       int rank = 0;
       for (int o = 0; o < groups; ++o) rank += o != g && (gs[o] > gs[g] || (gs[o] == gs[g] && o < g));
       if (rank >= keep)
         for (int j = 0; j < per; ++j) choice[g * per + j] = ninf;
     }
+    __syncthreads();
   }
   float sum = 0.f;
   for (int k = 0; k < top; ++k) {
-    int best = -1;
     float bv = ninf;
-    for (int e = 0; e < E; ++e) {
-      bool used = false;
-      for (int j = 0; j < k; ++j) used |= idx[j] == e;
-      if (used) continue;
-      if (best < 0 || choice[e] > bv) best = e, bv = choice[e];
+    int best = E;  // "none yet": any real index wins a tie against it
+    for (int e = lane; e < E; e += 64) {
+      const float c = choice[e];
+      if (c != c) continue;  // a NaN never ranks
+      if (best == E || c > bv) best = e, bv = c;  // ascending e: the lower index keeps a tie
     }
-    best = best < 0 ? 0 : best;
-    idx[k] = best;
-    float v = zr[best];
-    v = v == v ? v : 0.0f;
-    const float s = 1.0f / (1.0f + expf(-v));
-    wt[k] = s;
-    sum += s;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oi = __shfl_xor(best, o);
+      if (oi < E && (best == E || ov > bv || (ov == bv && oi < best))) bv = ov, best = oi;
+    }
+    best = best < E ? best : 0;
+    const float sg = score[best];
+    sum += sg;
+    __syncthreads();  // every lane has read choice[] for this pick
+    if (lane == 0) {
+      choice[best] = __builtin_nanf("");  // taken: out of every later pick
+      topk_idx[(int64_t)row * top + k] = best;
+      topk_w[(int64_t)row * top + k] = sg;
+    }
+    __syncthreads();
   }
   const float inv = scale / (sum + 1e-20f);
-  for (int k = 0; k < top; ++k) wt[k] *= inv;
+  __syncthreads();
+  for (int k = lane; k < top; k += 64) topk_w[(int64_t)row * top + k] *= inv;
 }
 
 inline int flat_blocks(int64_t n) {
@@ -191,17 +263,41 @@ inline int flat_blocks(int64_t n) {
 }  // namespace
 }  // namespace dsse
 
+namespace dsse {
+namespace {
+template <typename T, typename HT, int VEC>
+void launch_stream_mix(const StreamMixParams& p, hipStream_t st) {
+  const dim3 g(p.M), b(256);
+  switch (p.S) {
+    case 1: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 1, VEC>), g, b, 0, st, p); break;
+    case 2: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 2, VEC>), g, b, 0, st, p); break;
+    case 3: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 3, VEC>), g, b, 0, st, p); break;
+    case 4: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 4, VEC>), g, b, 0, st, p); break;
+    case 5: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 5, VEC>), g, b, 0, st, p); break;
+    case 6: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 6, VEC>), g, b, 0, st, p); break;
+    case 7: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 7, VEC>), g, b, 0, st, p); break;
+    default: hipLaunchKernelGGL((stream_mix_kernel<T, HT, 8, VEC>), g, b, 0, st, p); break;
+  }
+}
+template <int VEC>
+void launch_stream_mix_types(const StreamMixParams& p, hipStream_t st) {
+  if (p.f32) launch_stream_mix<float, float, VEC>(p, st);
+  else if (p.h_f32) launch_stream_mix<bf16, float, VEC>(p, st);
+  else launch_stream_mix<bf16, bf16, VEC>(p, st);
+}
+}  // namespace
+}  // namespace dsse
+
 extern "C" hipError_t dsse_stream_mix(const dsse::StreamMixParams* p, hipStream_t st) {
   if (p->M <= 0) return hipSuccess;
   if (p->S < 1 || p->S > dsse::kMaxStreams || p->nsum < 1) return hipErrorInvalidValue;
-  const dim3 g(p->M), b(256);
-  if (p->f32) {
-    hipLaunchKernelGGL((dsse::stream_mix_kernel<float, float>), g, b, 0, st, *p);
-  } else if (p->h_f32) {
-    hipLaunchKernelGGL((dsse::stream_mix_kernel<bf16, float>), g, b, 0, st, *p);
-  } else {
-    hipLaunchKernelGGL((dsse::stream_mix_kernel<bf16, bf16>), g, b, 0, st, *p);
-  }
+  // 16-byte accesses need every row of every operand on a 16-byte boundary: the width and the row stride multiples
+  // of four floats and the bases aligned (torch allocations are; column slices may not be)
+  auto al = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec = p->W % 4 == 0 && p->ld % 4 == 0 && al(p->streams) && al(p->y) && al(p->total) && al(p->norm_w) &&
+                   (p->h_f32 || p->f32 ? al(p->h) : true);
+  if (vec) dsse::launch_stream_mix_types<4>(*p, st);
+  else dsse::launch_stream_mix_types<1>(*p, st);
   return hipGetLastError();
 }
 
@@ -223,7 +319,7 @@ extern "C" hipError_t dsse_moe_route(const float* z, const float* corr, int M, i
                                      float scale, int* topk_idx, float* topk_w, hipStream_t st) {
   if (M <= 0) return hipSuccess;
   if (E > dsse::kMaxRouteExperts || groups < 1 || E % groups || top > E) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(dsse::moe_route_kernel, dim3((M + 63) / 64), dim3(64), 0, st, z, corr, M, E, top, groups, keep, scale,
+  hipLaunchKernelGGL(dsse::moe_route_kernel, dim3(M), dim3(64), 0, st, z, corr, M, E, top, groups, keep, scale,
                      topk_idx, topk_w);
   return hipGetLastError();
 }

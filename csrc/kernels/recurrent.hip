@@ -23,7 +23,7 @@ DEV float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
 DEV float softplusf(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
 DEV float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
 
-constexpr int kConvRows = 32;  // rows per workgroup of the convolution (its rows are independent of each other)
+constexpr int kConvRows = 8;   // rows per workgroup of the convolution (its rows are independent of each other)
 
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_kernel(ConvStateParams p) {
@@ -32,11 +32,12 @@ __global__ __launch_bounds__(256) void conv_state_kernel(ConvStateParams p) {
   const int ql = p.q_len[seq];
   const int t0 = blockIdx.z * kConvRows;
   if (c >= p.C || t0 >= ql) return;
-  const int t1 = t0 + kConvRows < ql ? t0 + kConvRows : ql;
+  // single: one launch block per sequence walks all of its rows (one, in a decode step) and then moves the tail itself
+  const int t1 = p.single ? ql : (t0 + kConvRows < ql ? t0 + kConvRows : ql);
   const int K = p.K, Kt = K - 1;
   const int row0 = p.q_start[seq];
   const bool fresh = p.ctx_len[seq] - ql == 0;  // the sequence starts in this step: nothing before it
-  const float* tail = p.tail + (int64_t)p.state_slot[seq] * Kt * p.C + c;  // tail[j * C]: input at offset j - Kt
+  float* tail = p.tail + (int64_t)p.state_slot[seq] * Kt * p.C + c;  // tail[j * C]: input at offset j - Kt
   const T* taps = reinterpret_cast<const T*>(p.taps) + (int64_t)c * K;
   const float bias = p.bias ? (float)reinterpret_cast<const T*>(p.bias)[c] : 0.0f;
   const float ib = p.in_bias ? (float)reinterpret_cast<const T*>(p.in_bias)[c] : 0.0f;  // the input projection's bias
@@ -50,9 +51,14 @@ __global__ __launch_bounds__(256) void conv_state_kernel(ConvStateParams p) {
     }
     if (p.act == 1) v = v / (1.0f + expf(-v));
     else if (p.act == 2) v += in[(int64_t)t * p.ld_in] + ib;
-    p.out[(int64_t)(row0 + t) * p.C + c] = v;
+    if (p.out) p.out[(int64_t)(row0 + t) * p.C + c] = v;
     if (p.out_b) reinterpret_cast<T*>(p.out_b)[(int64_t)(row0 + t) * p.C + c] = (T)v;
   }
+  if (p.single)  // this thread alone reads and writes its (slot, channel): ascending, as in conv_tail_kernel
+    for (int j = 0; j < Kt; ++j) {
+      const int i = ql - Kt + j;
+      tail[(int64_t)j * p.C] = i >= 0 ? in[(int64_t)i * p.ld_in] + ib : (fresh ? 0.0f : tail[(int64_t)(Kt + i) * p.C]);
+    }
 }
 
 // After every row of the step has read the old tail: the slot's new tail = the step's last K - 1 inputs.  Ascending:
@@ -198,14 +204,15 @@ __global__ __launch_bounds__(256) void lru_chunk_apply_kernel(LruScanParams p) {
 
 extern "C" hipError_t dsse_conv_state(const dsse::ConvStateParams* p, hipStream_t st) {
   if (p->nseq <= 0 || p->rows <= 0) return hipSuccess;
-  dim3 grid((p->C + 255) / 256, p->nseq, (p->rows + dsse::kConvRows - 1) / dsse::kConvRows);
+  dim3 grid((p->C + 255) / 256, p->nseq, p->single ? 1 : (p->rows + dsse::kConvRows - 1) / dsse::kConvRows);
   dim3 tgrid((p->C + 255) / 256, p->nseq);
+  const bool tails = p->K > 1 && !p->single;
   if (p->f32) {
     hipLaunchKernelGGL(dsse::conv_state_kernel<float>, grid, dim3(256), 0, st, *p);
-    if (p->K > 1) hipLaunchKernelGGL(dsse::conv_tail_kernel<float>, tgrid, dim3(256), 0, st, *p);
+    if (tails) hipLaunchKernelGGL(dsse::conv_tail_kernel<float>, tgrid, dim3(256), 0, st, *p);
   } else {
     hipLaunchKernelGGL(dsse::conv_state_kernel<bf16>, grid, dim3(256), 0, st, *p);
-    if (p->K > 1) hipLaunchKernelGGL(dsse::conv_tail_kernel<bf16>, tgrid, dim3(256), 0, st, *p);
+    if (tails) hipLaunchKernelGGL(dsse::conv_tail_kernel<bf16>, tgrid, dim3(256), 0, st, *p);
   }
   return hipGetLastError();
 }

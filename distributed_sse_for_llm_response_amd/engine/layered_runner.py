@@ -504,7 +504,7 @@ class LayeredRunner(RunnerBase):
 
     def _stream_buffers(self, M: int) -> dict:
         """Scratch of a step of M rows, each sized for the widest layer: `streams` the residual copies, `hn` a
-        sublayer's normed input and `hc` it after the input convolution (fp32), `big` the fused projection's fp32
+        sublayer's normed input before the input convolution (fp32), `big` the fused projection's fp32
         output, `cq` the normed query latent, `q` / `qabs` / `lat` the latent attention's operands, `o` a mixer's
         heads in fp32, `ao` them in the element type (the output projection's input), `up` / `h` the dense
         feed-forward's hidden row, and the routed experts' lists."""
@@ -528,7 +528,7 @@ class LayeredRunner(RunnerBase):
                 else:
                     ff = max(ff, L.mlp.ff)
         d = {"streams": torch.zeros(M, cfg.num_streams, W, **f32), "hn": torch.zeros(M, W, **f32),
-             "hc": torch.zeros(M, W, **f32), "big": torch.zeros(M * big, **f32), "cq": torch.zeros(M * cq, **el),
+             "big": torch.zeros(M * big, **f32), "cq": torch.zeros(M * cq, **el),
              "q": torch.zeros(M * q, **el), "qabs": torch.zeros(M * qabs, **f32), "lat": torch.zeros(M * qabs, **el),
              "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32), "ao": torch.zeros(M * o, **el),
              "up": torch.zeros(M * ff, **f32), "h": torch.zeros(M * ff, **el)}
@@ -568,7 +568,7 @@ class LayeredRunner(RunnerBase):
                 if conv:
                     for g in groups:
                         ops.conv_state(d["hn"], hc.canon, None, self.state.tail.get((run.index, sub)), g["qs"], g["ql"],
-                                       g["ctx"], g["ss"], d["hc"], d["xb"], None, 2)
+                                       g["ctx"], g["ss"], None, d["xb"], None, 2, g["qt"] == 1)
                 if sub == 1:
                     getattr(self, "_" + L.kind + "_streams")(run.index, L.mixer, Lw.mix, M, d, pos, slots, groups)
                     prev = (d["y"], 1, hc)
@@ -686,7 +686,7 @@ class LayeredRunner(RunnerBase):
         r = slice(0, B)
         ops.decode_prep(self.active[r], self.positions[r], self.block_tables[r], self.slots[r], self.ctx_len[r],
                         self.q_len[r], self.kv.num_blocks)
-        d = {k: (v[:B] if k in ("resid", "xb", "y", "y2", "streams", "hn", "hc") else v) for k, v in self._dec.items()}
+        d = {k: (v[:B] if k in ("resid", "xb", "y", "y2", "streams", "hn") else v) for k, v in self._dec.items()}
         self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
         self._head(d["resid"], self._dec["xb"][:B], self.logits[r])
         self._sample_commit(B)

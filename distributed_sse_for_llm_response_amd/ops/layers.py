@@ -79,13 +79,16 @@ def latent_attention(q, q_abs, cache, block_tables, q_start, q_len, ctx_len, wor
                               window, scale, qt, vt)
 
 
-def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None, act: int = 0):
+def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias=None, act: int = 0,
+               single: bool = False):
     """Per-channel causal convolution continued from each sequence's slot tail (and the tail's update); in_bias is
     added to every input (the bias of the projection that made `inp`).  `inp` may be a column slice of a wider fp32
-    buffer; bias and out_b (the output once more in the element type) may be None; act 1 applies SiLU to the output, act 2
-    adds the row's own input to it (inp + conv(inp))."""
+    buffer; bias, out (fp32) and out_b (the output in the element type) may be None (not both outputs); act 1 applies
+    SiLU to the output, act 2 adds the row's own input to it (inp + conv(inp)).  single: every sequence of the call has
+    one row (a decode step), so one launch also moves the tails."""
     if _hip(inp):
-        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias, act)
+        torch.ops.dsse.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias, act,
+                                  single)
     else:
         lref.conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, out_b, in_bias, act)
 

@@ -125,7 +125,8 @@ def conv_state(inp, taps, bias, tail, q_start, q_len, ctx_len, state_slot, out, 
             y = torch.nn.functional.silu(y)
         elif act == 2:
             y = y + seq[K - 1:]
-        out[r0:r0 + ql] = y
+        if out is not None:
+            out[r0:r0 + ql] = y
         if out_b is not None:
             out_b[r0:r0 + ql] = y.to(out_b.dtype)
         if K > 1:

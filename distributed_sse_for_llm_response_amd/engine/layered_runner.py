@@ -504,7 +504,8 @@ class LayeredRunner(RunnerBase):
 
     def _stream_buffers(self, M: int) -> dict:
         """Scratch of a step of M rows, each sized for the widest layer: `streams` the residual copies, `hn` a
-        sublayer's normed input before the input convolution (fp32), `big` the fused projection's fp32
+        sublayer's normed input before the input convolution and `hc` after it (fp32; the latter only where a router
+        reads it), `big` the fused projection's fp32
         output, `cq` the normed query latent, `q` / `qabs` / `lat` the latent attention's operands, `o` a mixer's
         heads in fp32, `ao` them in the element type (the output projection's input), `up` / `h` the dense
         feed-forward's hidden row, and the routed experts' lists."""
@@ -528,7 +529,7 @@ class LayeredRunner(RunnerBase):
                 else:
                     ff = max(ff, L.mlp.ff)
         d = {"streams": torch.zeros(M, cfg.num_streams, W, **f32), "hn": torch.zeros(M, W, **f32),
-             "big": torch.zeros(M * big, **f32), "cq": torch.zeros(M * cq, **el),
+             "hc": torch.zeros(M, W, **f32) if moe else None, "big": torch.zeros(M * big, **f32), "cq": torch.zeros(M * cq, **el),
              "q": torch.zeros(M * q, **el), "qabs": torch.zeros(M * qabs, **f32), "lat": torch.zeros(M * qabs, **el),
              "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32), "ao": torch.zeros(M * o, **el),
              "up": torch.zeros(M * ff, **f32), "h": torch.zeros(M * ff, **el)}
@@ -561,19 +562,22 @@ class LayeredRunner(RunnerBase):
                     continue
                 y, nsum, pw = prev if prev else (None, 1, None)
                 conv = hc.canon is not None and hc.canon.shape[1] > 0
+                routed = sub == 2 and hasattr(L.mlp, "experts")  # the router reads the fp32 row, not its rounding
                 ops.stream_mix(y, nsum, mult, x, ids if first else None, w.embed if first else None, cfg.embed_scale,
                                pw.outw if pw else None, pw.mix if pw else None, hc.inw, hc.norm, eps,
-                               d["hn"] if conv else d["xb"])
+                               d["hn"] if conv or routed else d["xb"])
                 first = False
                 if conv:
                     for g in groups:
                         ops.conv_state(d["hn"], hc.canon, None, self.state.tail.get((run.index, sub)), g["qs"], g["ql"],
-                                       g["ctx"], g["ss"], None, d["xb"], None, 2, g["qt"] == 1)
+                                       g["ctx"], g["ss"], d["hc"] if routed else None, d["xb"], None, 2, g["qt"] == 1)
+                elif routed:
+                    ops.act_rows(d["hn"], d["xb"], 0)
                 if sub == 1:
                     getattr(self, "_" + L.kind + "_streams")(run.index, L.mixer, Lw.mix, M, d, pos, slots, groups)
                     prev = (d["y"], 1, hc)
-                elif hasattr(L.mlp, "experts"):
-                    prev = self._routed_ff(L.mlp, Lw.mlp, M, d) + (hc,)
+                elif routed:
+                    prev = self._routed_ff(L.mlp, Lw.mlp, M, d, d["hc"] if conv else d["hn"]) + (hc,)
                 else:
                     self._act_ff(L.mlp, Lw.mlp, M, d)
                     prev = (d["y"], 1, hc)
@@ -661,14 +665,15 @@ class LayeredRunner(RunnerBase):
         ops.act_rows(up, h, 1, Fw.act)
         self._lin(h, Fw.down, Fw.down_t, d["y"])
 
-    def _routed_ff(self, f, Fw, M: int, d: dict):
-        """Router GEMM (fp32 logits) -> group-limited sigmoid routing -> grouped squared-ReLU experts; returns
+    def _routed_ff(self, f, Fw, M: int, d: dict, h32):
+        """Router GEMM in true fp32 on the sublayer's fp32 input `h32` (a close call is decided by the row itself, not by
+        its rounding) -> group-limited sigmoid routing -> grouped squared-ReLU experts on the element-type row; returns
         (per-slot outputs [M * top, W] fp32, top): the stream step that follows sums them."""
         tki = d["tki"][:M * f.top].view(M, f.top)
         tkw = d["tkw"][:M * f.top].view(M, f.top)
         o = d["mo_o"][:M * f.top * self.cfg.width].view(M * f.top, self.cfg.width)
         z = d["mo_z"][:M * f.experts].view(M, f.experts)
-        ops.gemm_rm(d["xb"], Fw.router, z)
+        ops.gemm_rm(h32, Fw.router, z)
         ops.moe_route(z, Fw.correction, tki, tkw, f.groups, f.keep, f.scale)
         ops.moe_grouped(d["xb"], tki, tkw, None, Fw.up, Fw.down, None, None, None, d["mo_sorted"], d["mo_tile"],
                         d["mo_n"], d["mo_h"], o)
@@ -686,7 +691,8 @@ class LayeredRunner(RunnerBase):
         r = slice(0, B)
         ops.decode_prep(self.active[r], self.positions[r], self.block_tables[r], self.slots[r], self.ctx_len[r],
                         self.q_len[r], self.kv.num_blocks)
-        d = {k: (v[:B] if k in ("resid", "xb", "y", "y2", "streams", "hn") else v) for k, v in self._dec.items()}
+        rows = ("resid", "xb", "y", "y2", "streams", "hn", "hc")
+        d = {k: (v[:B] if k in rows and v is not None else v) for k, v in self._dec.items()}
         self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
         self._head(d["resid"], self._dec["xb"][:B], self.logits[r])
         self._sample_commit(B)

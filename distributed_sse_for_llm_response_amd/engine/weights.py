@@ -565,7 +565,7 @@ class ActFfWeights:
 
 @dataclass
 class RoutedFfWeights:
-    router: torch.Tensor     # [E, W]
+    router: torch.Tensor     # [E, W] fp32 in both element types (the router runs in true fp32 on the fp32 row)
     correction: torch.Tensor  # [E] fp32
     up: torch.Tensor         # [E, F, W]
     down: torch.Tensor       # [E, W, F]
@@ -655,7 +655,7 @@ def convert_dironex(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> L
                 _tile_fields(layer.mlp, ("up", "down"))
             else:
                 stack = lambda leaf: torch.stack([t(f"{p}mlp.e{e}.{leaf}") for e in range(fs.experts)]).contiguous()  # noqa: E731
-                layer.mlp = RoutedFfWeights(router=t(p + "mlp.router"), correction=f(p + "mlp.correction"),
+                layer.mlp = RoutedFfWeights(router=f(p + "mlp.router"), correction=f(p + "mlp.correction"),
                                             up=stack("up"), down=stack("down"))
         layers.append(layer)
     out = LayeredWeights(cfg=cfg, embed=t("embed"), layers=layers, final_norm=f("final.norm"), head=t("head"),

@@ -1,6 +1,7 @@
-"""Forward passes of configuration-driven designs (models/muderax.py, models/surodra.py) on the layer-mechanism kernels
-(ops/layers.py).  Two block styles share the runner: sandwich norms on a sublayer's output (Muderax, described first)
-and pre-norm blocks around matrix-state mixers (Surodra, described after it).
+"""Forward passes of configuration-driven designs (models/muderax.py, models/surodra.py, models/dironex.py) on the
+layer-mechanism kernels (ops/layers.py).  Three block styles share the runner: sandwich norms on a sublayer's output
+(Muderax, described first), pre-norm blocks around matrix-state mixers (Surodra, described after it) and pre-norm
+blocks on several residual streams (Dironex, described last).
 
 A step is a set of packed rows -- the B decode slots first (one row each, state on the device as in ModelRunner), then
 the rows of prompt portions -- that walk the layer list once:
@@ -37,10 +38,27 @@ same weights and its own pages and state slots per pass:
 
 Long prompt groups walk the recurrences without the delta rule in two levels (matrix_scan_chunked).
 
+The multi-stream walk (`_stream_layers`) also goes over layer runs; a row carries S residual copies:
+
+    stream_mix              (first step) every stream = embedding * scale; x_t = sum_s mix[s][t] x_s + m out[t] y for the
+                            finished sublayer; u = sum_s in[s] x_s; RMS norm with a gain per channel -- one kernel
+    conv_state (act 2)      h + conv(h) over time per channel, continued from the slot's tail of normed rows (one launch
+                            for decode rows, rows in parallel + a tail kernel for prompt portions)
+    latent attention        ONE fused GEMM [dq | dkv | g] (fp32 out) -> stream_mix as the query latent's RMS norm -> query
+                            up-projection -> latent_kv_write from the dkv columns -> per-head fold -> latent_attention
+                            (causal, this run's latent pages) -> per-head value up-projection (fp32) -> act_rows (times
+                            sigmoid(g)) -> output GEMM
+    windowed attention      fused GEMM [q | k | v] -> norm_rope_rows kind 3 (RMS per head; k and v into this run's pages)
+                            -> sink_attention without sink and gate over the window -> output GEMM
+    feed-forward            up GEMM -> act_rows (xIELU) -> down GEMM; or router GEMM in fp32 on the fp32 row -> moe_route
+                            (group-limited sigmoid routing) -> moe_grouped without a gate (squared ReLU), per-slot outputs
+                            summed inside the next stream_mix
+    head                    stream_mix (last write-back, sum of the streams) -> RMS norm -> head GEMM
+
 The residual stream, norms, scores, router and recurrence are fp32 in both element types; ``dtype=torch.float32`` runs
 the projections in true fp32 as well (the exact mode).  The cache is paged with the engine's block tables and
-allocator (LatentKVCache, PagedKVCache); recurrent layers keep their state in the sequence's decode slot
-(RecurrentStateCache, MatrixStateCache), so
+allocator (LatentKVCache, PagedKVCache, both at once in MixedKVCache); recurrent layers and input convolutions keep
+their state in the sequence's decode slot (RecurrentStateCache, MatrixStateCache, ConvTailCache), so
 slots and pages are handed from one sequence to the next with no clearing pass.  The decode step of each batch bucket
 is captured into a graph like ModelRunner's; prompt portions and mixed steps run eagerly.
 """

@@ -1,5 +1,6 @@
 """Plain-PyTorch references of the layer-mechanism ops (``ops/layers.py``): exact semantics of the HIP kernels in
-``csrc/kernels/{gemm_rowmajor,norms,latent_attention,recurrent,moe}.hip``, including the cache and state layouts.
+``csrc/kernels/{gemm_rowmajor,norms,latent_attention,recurrent,moe,stream_ops,sink_attention,matrix_scan,multistream}.hip``,
+including the cache and state layouts.
 
 As with ``ops/reference.py`` they are the numerics oracle of the kernel tests and the CPU execution path of the engine
 (scheduler, cache and state-slot plumbing run here without a GPU).  Everything is computed in fp32 on whatever element

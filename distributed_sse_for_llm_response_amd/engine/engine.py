@@ -649,7 +649,8 @@ class LLMEngine:
                 s.admit_ns = time.time_ns()
             last = s.prefilled + n == len(s.prompt)
             chunks.append(PrefillSeq(slot=s.slot, tokens=s.prompt[s.prefilled:s.prefilled + n], start_pos=s.prefilled,
-                                     block_table=s.blocks, last_chunk=last))
+                                     block_table=s.blocks, last_chunk=last,
+                                     prev_token=s.prompt[s.prefilled - 1] if s.prefilled > 0 else -1))
             s.prefilled += n
             budget -= n
             if last:
@@ -871,7 +872,8 @@ class LLMEngine:
             else:
                 s.state = "prefill"
                 chunks.append(PrefillSeq(slot=s.slot, tokens=list(tokens), start_pos=pos0, block_table=s.blocks,
-                                         last_chunk=False, want=tuple(int(o) for o in want)))
+                                         last_chunk=False, want=tuple(int(o) for o in want),
+                                         prev_token=int(s.prompt[pos0 - 1]) if pos0 > 0 else -1))
                 order.append(("c", len(chunks) - 1, len(want)))
             s.prefilled = pos0 + n
         # sequences left out of this step hold: not in the decode rows (their slots stay inactive)

@@ -71,7 +71,7 @@ import torch
 
 from .. import ops
 from ..models.muderax import LRU_DECAY_SCALE
-from ..models.surodra import UNIT_EPS
+from ..models.surodra import UNIT_EPS, HalfRotarySpec
 from ..parallel.comm import TPComm
 from .kv_cache import (PAGE, ConvTailCache, LatentKVCache, MatrixStateCache, MixedKVCache, PagedKVCache,
                        RecurrentStateCache)
@@ -104,7 +104,10 @@ class LayeredRunner(RunnerBase):
         self.num_blocks = num_blocks
         self.prenorm = getattr(cfg, "family", "") == "surodra"   # pre-norm blocks with matrix-state mixers
         self.multistream = getattr(cfg, "family", "") == "dironex"  # pre-norm blocks on several residual streams
-        if self.multistream:
+        self.bracket = getattr(cfg, "family", "") == "murulorn"    # a norm before and after each sublayer, token inputs
+        if self.bracket:
+            self._setup_bracket()
+        elif self.multistream:
             self._setup_streams()
         elif self.prenorm:
             self._setup_prenorm()
@@ -159,6 +162,9 @@ class LayeredRunner(RunnerBase):
         el = dict(device=dev, dtype=self.dtype)
         W = cfg.width
         d = {"resid": torch.zeros(M, W, **f32), "xb": torch.zeros(M, W, **el), "y": torch.zeros(M, W, **f32)}
+        if self.bracket:
+            d.update(self._bracket_buffers(M))
+            return d
         if self.multistream:
             d.update(self._stream_buffers(M))
             return d
@@ -281,11 +287,16 @@ class LayeredRunner(RunnerBase):
                         d["mo_tile"], d["mo_n"], d["mo_h"], o)
         return o, S
 
-    def _layers(self, M: int, d: dict, ids, pos, slots, groups: list, trace: list | None = None) -> None:
+    def _layers(self, M: int, d: dict, ids, pos, slots, groups: list, trace: list | None = None, prev=None) -> None:
         """Embedding + every layer over M packed rows.  `groups`: sequence groups of the step (decode slots, prompt
         portions), each with its own metadata (block tables bt, q_start qs, q_len ql, ctx_len ctx, state slots ss,
-        attention work items ws / wt of qt rows).  trace (a list) receives a copy of the stream after every layer."""
+        attention work items ws / wt of qt rows).  trace (a list) receives a copy of the stream after every layer.
+        prev: (previous token per row, where decode rows store their own token, which of them do) for designs whose
+        embedding reads the previous token."""
         cfg, eps = self.cfg, self.cfg.eps
+        if self.bracket:
+            self._bracket_layers(M, d, ids, prev, pos, slots, groups, trace)
+            return
         if self.multistream:
             self._stream_layers(M, d, ids, pos, slots, groups, trace)
             return
@@ -312,7 +323,10 @@ class LayeredRunner(RunnerBase):
         self._head(rows, xn, logits)
 
     def _head(self, resid, xn, logits) -> None:
-        if self.multistream:  # resid holds the sum of the streams: one stream with weight 1 through the RMS norm
+        if self.bracket:
+            ops.add_norm_rows(None, 1, None, resid, self.w.final_norm, self.cfg.eps, xn)
+            self._lin(xn, self.w.head, self.w.head_t, logits)
+        elif self.multistream:  # resid holds the sum of the streams: one stream with weight 1 through the RMS norm
             ops.stream_mix(None, 1, 0.0, resid.unsqueeze(1), in_w=self.w.ones[:1], norm_w=self.w.final_norm,
                            eps=self.cfg.eps, h=xn)
             self._lin(xn, self.w.head, self.w.head_t, logits)
@@ -697,6 +711,219 @@ class LayeredRunner(RunnerBase):
                         d["mo_n"], d["mo_h"], o)
         return o, f.top
 
+
+    # ------------------------------------------------------------------ bracketing norms, token inputs, rotated values
+    def _setup_bracket(self) -> None:
+        """Caches and state of a design with bracketing norms, keyed by layer RUN: keys and values (the values rotated
+        by their positions) for the attention runs, matrix state and convolution tail for the channel-delta runs, and
+        every slot's previous token (the hashed bigram embedding reads it)."""
+        cfg, dev = self.cfg, self.device
+        self.runs = cfg.runs()
+        kv, st, self._rope = {}, {}, {}
+        for r in self.runs:
+            L, m = cfg.layers[r.layer], cfg.layers[r.layer].mixer
+            if L.kind == "attention":
+                kv[r.index] = (m.kv_heads, m.dim, m.vdim)
+                for dims in (m.rot_dims, m.vdim):
+                    rot = HalfRotarySpec(dims=dims, base=m.rot_base)
+                    if dims > 0 and rot not in self._rope:
+                        self._rope[rot] = rot.table(self.max_model_len + 1, dev)
+            else:
+                st[r.index] = ((m.heads, m.dim, m.vdim), 2 * m.kv_heads * m.dim + m.heads * m.vdim, m.conv)
+        # the MFMA form turns a head's output back inside its registers: both halves of a pair must be whole tiles
+        flash = [r for r, (_, dm, v) in kv.items() if ops.sink_flash_ok(self.dtype, dm, v) and v % 32 == 0]
+        self.kv = PagedKVCache(kv, self.num_blocks, dev, self.dtype, transposed=flash)
+        self.state = MatrixStateCache(st, self.max_batch, dev)
+        self.prev_ids = torch.zeros(self.max_batch, device=dev, dtype=torch.int32)
+        self._host_prev = {}  # slot -> last token of the latest prompt portion (when the caller names no predecessor)
+
+    def _bracket_buffers(self, M: int) -> dict:
+        """Scratch of a step of M rows, each sized for the widest layer: `big` the fused projection's fp32 output, `cv`
+        the convolution's, `z` the per-channel decays, `gz` the output gate's pre-activations, `qa` the attention's
+        normed and rotated queries, `o` the recurrence's heads, `ao` a mixer's gated output in the element type, `up` /
+        `h` the dense feed-forward's hidden row, `hn` the fp32 normed row a router reads, `cat` [stream | embedding
+        output] for the projection that opens a loop pass, `sg` / `sh` the token input's gate, and the experts' lists."""
+        from ..models.murulorn import SoftmaxRoutedSpec
+
+        cfg, dev = self.cfg, self.device
+        f32 = dict(device=dev, dtype=torch.float32)
+        el = dict(device=dev, dtype=self.dtype)
+        W = cfg.width
+        big = cv = z = gz = qa = o = ff = 1
+        moe = []
+        for i, L in enumerate(cfg.layers):
+            m = L.mixer
+            big = max(big, self.w.layers[i].mix.n_big)
+            o = max(o, m.heads * m.vdim)
+            if L.kind == "attention":
+                qa = max(qa, m.heads * m.dim)
+            else:
+                cv, z = max(cv, 2 * m.kv_heads * m.dim + m.heads * m.vdim), max(z, m.heads * m.dim)
+                gz = max(gz, m.heads * m.vdim)
+            if isinstance(L.mlp, SoftmaxRoutedSpec):
+                moe.append(L.mlp)
+            elif L.mlp is not None:
+                ff = max(ff, L.mlp.ff)
+        d = {"big": torch.zeros(M * big, **f32), "cv": torch.zeros(M * cv, **f32), "z": torch.zeros(M * z, **f32),
+             "gz": torch.zeros(M * gz, **f32), "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32),
+             "ao": torch.zeros(M * o, **el), "up": torch.zeros(M * ff, **f32), "h": torch.zeros(M * ff, **el),
+             "hn": torch.zeros(M, W, **f32) if moe else None,
+             "cat": torch.zeros(M, 2 * W, **el) if cfg.loop_times > 0 else None,
+             "sg": torch.zeros(M * max(1, cfg.side_dim), **f32), "sh": torch.zeros(M * max(1, cfg.side_dim), **el)}
+        if moe:
+            top = max(f.top for f in moe)
+            tiles = -(-M * top // 64) + max(f.experts for f in moe) + 2
+            ldh = -(-max(f.ff for f in moe) // 8) * 8
+            d.update({"tki": torch.zeros(M * top, device=dev, dtype=torch.int32), "tkw": torch.zeros(M * top, **f32),
+                      "mo_z": torch.zeros(M * max(f.experts for f in moe), **f32),
+                      "mo_sorted": torch.zeros(tiles * 64, device=dev, dtype=torch.int32),
+                      "mo_tile": torch.zeros(tiles, device=dev, dtype=torch.int32),
+                      "mo_n": torch.zeros(1, device=dev, dtype=torch.int32), "mo_h": torch.zeros(M * top, ldh, **el),
+                      "mo_o": torch.zeros(M * top * W, **f32)})
+        return d
+
+    def _bracket_layers(self, M: int, d: dict, ids, prev, pos, slots, groups: list, trace: list | None) -> None:
+        """Every layer run over M packed rows.  Between sublayers ONE add_norm_rows adds the finished sublayer's normed
+        output to the stream and norms the stream for the next one (or rounds it, for the token input's gate and for
+        the projection that opens a loop pass); the last output is added before the head's norm.  `pending` is the
+        sublayer output that is not in the stream yet: (rows, parts per row, gain of its norm)."""
+        from ..models.murulorn import SoftmaxRoutedSpec
+
+        cfg, w, eps = self.cfg, self.w, self.cfg.eps
+        W = cfg.width
+        bg = cfg.bigram
+        prev_rows, prev_out, keep = prev if prev is not None else (None, None, None)
+        if bg is not None and prev_rows is None:
+            raise ValueError(f"{cfg.name}: the embedding reads each row's previous token")
+        cat = d["cat"]
+        ops.embed_pair_rows(ids, prev_rows, pos, w.embed, w.bigram, bg.mul_prev if bg else 0, bg.mul_cur if bg else 0,
+                            bg.buckets if bg else 1, d["resid"], cat[:, W:] if cat is not None else None, prev_out, keep)
+        pending = (None, 1, None)
+        for run in self.runs:
+            L, Lw = cfg.layers[run.layer], w.layers[run.layer]
+            if run.pass_no >= 0:  # a pass of the looped span opens: stream <- W_in [stream | embedding output]
+                ops.add_norm_rows(*pending, d["resid"], None, eps, cat[:, :W])
+                self._lin(cat, w.loop_in, w.loop_in_t, d["resid"])
+                pending = (None, 1, None)
+            ops.add_norm_rows(*pending, d["resid"], Lw.norm1, eps, d["xb"])
+            getattr(self, "_" + L.kind + "_bracket")(run.index, L.mixer, Lw.mix, M, d, pos, slots, groups)
+            pending = (d["y"], 1, Lw.norm1b)
+            if L.mlp is not None:
+                routed = isinstance(L.mlp, SoftmaxRoutedSpec)
+                ops.add_norm_rows(*pending, d["resid"], Lw.norm2, eps, d["xb"], d["hn"] if routed else None)
+                if routed:
+                    pending = self._softmax_routed_ff(L.mlp, Lw.mlp, M, d) + (Lw.norm2b,)
+                else:
+                    self._relu2_ff(L.mlp, Lw.mlp, M, d)
+                    pending = (d["y"], 1, Lw.norm2b)
+            if Lw.side is not None:  # the layer's token input reads the stream after the feed-forward
+                sd = Lw.side
+                F = sd.gate.shape[0]
+                sg, sh = d["sg"][:M * F].view(M, F), d["sh"][:M * F].view(M, F)
+                ops.add_norm_rows(*pending, d["resid"], None, eps, d["xb"])
+                ops.gemm_rm(d["xb"], sd.gate, sg)
+                ops.token_gate_rows(sg, ids, w.side_embed, sd.col0, sh)
+                ops.gemm_rm(sh, sd.proj, d["y"])
+                pending = (d["y"], 1, sd.norm)
+            if trace is not None:
+                ops.add_norm_rows(*pending, d["resid"], None, eps)
+                pending = (None, 1, None)
+                trace.append(d["resid"].clone())
+        if pending[0] is not None:
+            ops.add_norm_rows(*pending, d["resid"], None, eps)
+
+    def _attention_bracket(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        """Softmax attention whose values are rotated by their positions: ONE fused GEMM [q | k | v | g] (fp32 out) ->
+        norm rows (q: whole-row RMS norm + rotation into a buffer; k the same into this run's pages; v: RMS norm per
+        head + rotation over the whole value width into the pages, also transposed) -> attention over the window with
+        capped scores, each head's sum turned back by the row's position and gated -> output GEMM."""
+        H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
+        big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        kc, vc, vt = self.kv.k[ri], self.kv.v[ri], self.kv.vt.get(ri)
+        rope = self._rope.get(HalfRotarySpec(dims=m.rot_dims, base=m.rot_base))
+        vrope = self._rope[HalfRotarySpec(dims=V, base=m.rot_base)]
+        qa = d["qa"][:M * H * D].view(M, H, D)
+        eps = self.cfg.eps
+        ops.norm_rope_rows(self._cols(big, 0, H, D), Lw.q_norm, pos, rope, qa, None, 1, eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, H * D, G, D), Lw.k_norm, pos, rope, kc, slots, 1, eps, 1.0)
+        ops.norm_rope_rows(self._cols(big, (H + G) * D, G, V), None, pos, vrope, vc, slots, 3, eps, 1.0, vt)
+        gate = big[:, (H + G) * D + G * V:(H + G) * D + G * V + H]
+        ao = d["ao"][:M * H * V].view(M, H, V)
+        for g in groups:
+            if vt is not None and g["qt"] > 1:
+                ops.sink_attention(qa, kc, vc, g["bt"], g["qs"], g["ql"], g["ctx"], g["hs"], g["ht"], None, gate, ao,
+                                   m.window, m.scale, SINK_ROWS_TILE, vt, False, m.softcap, vrope)
+            elif vt is not None and V <= ops.layers.SINK_SPLIT_MAX_V:
+                ops.sink_attention(qa, kc, vc, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], None, gate, ao,
+                                   m.window, m.scale, SINK_ROWS_TILE, vt, True, m.softcap, vrope)
+            else:
+                ops.sink_attention(qa, kc, vc, g["bt"], g["qs"], g["ql"], g["ctx"], g["ws"], g["wt"], None, gate, ao,
+                                   m.window, m.scale, g["qt"], None, False, m.softcap, vrope)
+        self._lin(ao.view(M, H * V), Lw.o, Lw.o_t, d["y"])
+
+    def _channel_delta_bracket(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
+        """Gated delta rule with a decay per head and key channel: ONE fused GEMM [q | k | v | b | a1 | g1] (fp32 out)
+        -> conv_state over q | k | v (SiLU; slot tail) -> unit q, k per head -> the decay's and the gate's second
+        projections in fp32 -> gate_math (one rate per head, one bias per head and channel) -> matrix_scan (delta rule
+        with per-channel decay; slot state) -> per-head RMS norm times the sigmoid gate -> output GEMM."""
+        H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
+        C = 2 * G * D + H * V
+        ra, rg = Lw.a2.shape[1], Lw.g2.shape[1]
+        big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
+        cv = d["cv"][:M * C].view(M, C)
+        self._lin(d["xb"], Lw.big, Lw.big_t, big)
+        for g in groups:
+            ops.conv_state(big[:, :C], Lw.conv, None, self.state.tail.get(ri), g["qs"], g["ql"], g["ctx"], g["ss"], cv,
+                           None, None, 1)
+        q, k, v = self._cols(cv, 0, G, D), self._cols(cv, G * D, G, D), self._cols(cv, 2 * G * D, H, V)
+        ops.norm_rope_rows(q, None, pos, None, q, None, 2, UNIT_EPS, D ** -0.5)
+        ops.norm_rope_rows(k, None, pos, None, k, None, 2, UNIT_EPS, 1.0)
+        beta = big[:, C:C + H]
+        ops.gate_math(beta, 1)
+        z = d["z"][:M * H * D].view(M, H * D)
+        gz = d["gz"][:M * H * V].view(M, H * V)
+        ops.gemm_rm(big[:, C + H:C + H + ra], Lw.a2, z)
+        ops.gate_math(z, 0, Lw.a_log, Lw.dt_bias)
+        ops.gemm_rm(big[:, C + H + ra:C + H + ra + rg], Lw.g2, gz)
+        o = d["o"][:M * H * V].view(M, H, V)
+        for g in groups:
+            ops.matrix_scan(q, k, v, z.view(M, H, D), beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"], o,
+                            1.0)
+        ao = d["ao"][:M * H * V].view(M, H * V)
+        ops.gated_head_norm(o, Lw.norm, gz, self.cfg.eps, ao, 1)
+        self._lin(ao, Lw.o, Lw.o_t, d["y"])
+
+    def _relu2_ff(self, f, Fw, M: int, d: dict) -> None:
+        """Dense feed-forward: up GEMM (fp32) -> squared ReLU -> down GEMM."""
+        up = d["up"][:M * f.ff].view(M, f.ff)
+        h = d["h"][:M * f.ff].view(M, f.ff)
+        self._lin(d["xb"], Fw.up, Fw.up_t, up)
+        ops.act_rows(up, h, 2)
+        self._lin(h, Fw.down, Fw.down_t, d["y"])
+
+    def _softmax_routed_ff(self, f, Fw, M: int, d: dict):
+        """Router GEMM in true fp32 on the fp32 normed row -> softmax scores, group-limited choice, unnormalised weights
+        -> grouped squared-ReLU experts on the element-type row; returns (per-slot outputs [M * top, W] fp32, top): the
+        add_norm_rows that follows sums them."""
+        tki = d["tki"][:M * f.top].view(M, f.top)
+        tkw = d["tkw"][:M * f.top].view(M, f.top)
+        o = d["mo_o"][:M * f.top * self.cfg.width].view(M * f.top, self.cfg.width)
+        z = d["mo_z"][:M * f.experts].view(M, f.experts)
+        ops.gemm_rm(d["hn"], Fw.router, z)
+        ops.moe_route(z, None, tki, tkw, f.groups, f.keep, 1.0, 1)
+        ops.moe_grouped(d["xb"], tki, tkw, None, Fw.up, Fw.down, None, None, None, d["mo_sorted"], d["mo_tile"],
+                        d["mo_n"], d["mo_h"], o)
+        return o, f.top
+
+    def _remember_last(self, seqs: list, g: dict) -> None:
+        """After prompt portions: every portion's last token becomes its slot's previous token."""
+        if not self.bracket:
+            return
+        self.prev_ids.index_copy_(0, g["ss"].long(), g["last"])
+        for s in seqs:
+            self._host_prev[s.slot] = int(s.tokens[-1])
+
     # ------------------------------------------------------------------ decode
     def _decode_group(self, B: int) -> dict:
         r = slice(0, B)
@@ -709,9 +936,10 @@ class LayeredRunner(RunnerBase):
         r = slice(0, B)
         ops.decode_prep(self.active[r], self.positions[r], self.block_tables[r], self.slots[r], self.ctx_len[r],
                         self.q_len[r], self.kv.num_blocks)
-        rows = ("resid", "xb", "y", "y2", "streams", "hn", "hc")
+        rows = ("resid", "xb", "y", "y2", "streams", "hn", "hc", "cat")
         d = {k: (v[:B] if k in rows and v is not None else v) for k, v in self._dec.items()}
-        self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)])
+        prev = (self.prev_ids[r], self.prev_ids[r], self.q_len[r]) if self.bracket else None
+        self._layers(B, d, self.ids[r], self.positions[r], self.slots[r], [self._decode_group(B)], prev=prev)
         self._head(d["resid"], self._dec["xb"][:B], self.logits[r])
         self._sample_commit(B)
         ops.ring_advance(self.ring_counter)
@@ -749,6 +977,10 @@ class LayeredRunner(RunnerBase):
         if self.device.type == "cuda":
             idx = idx.pin_memory().to(self.device, non_blocking=True)
         self.state.move(idx[0], idx[1])
+        if self.bracket:
+            self.prev_ids.index_copy_(0, idx[1], self.prev_ids.index_select(0, idx[0]))
+            moved = {b: self._host_prev.get(a) for a, b in zip(src, dst)}
+            self._host_prev.update({b: t for b, t in moved.items() if t is not None})
 
     def close(self) -> None:
         pass
@@ -760,6 +992,7 @@ class LayeredRunner(RunnerBase):
         n = len(seqs)
         ids_l, pos_l, slots_l, qs, ql, ctx, ss = [], [], [], [], [], [], []
         ws, wt, fs, ft, hs, ht = [], [], [], [], [], []
+        prev_l, last = [], []
         bt = torch.zeros(n, self.max_blocks, dtype=torch.int32)
         row = 0
         for i, s in enumerate(seqs):
@@ -767,6 +1000,15 @@ class LayeredRunner(RunnerBase):
             p = s.start_pos + np.arange(m, dtype=np.int64)
             table = np.asarray(s.block_table, dtype=np.int64)
             ids_l.append(np.asarray(s.tokens, dtype=np.int64))
+            if self.bracket:  # each row's previous token: the caller's (or the slot's remembered one), then the portion's own
+                first = -1
+                if s.start_pos > 0:
+                    first = s.prev_token if s.prev_token >= 0 else self._host_prev.get(s.slot, -1)
+                    if first < 0:
+                        raise ValueError(f"slot {s.slot}: a portion that starts at position {s.start_pos} needs the token "
+                                         "before it (PrefillSeq.prev_token)")
+                prev_l.append(np.concatenate([[first], ids_l[-1][:-1]]).astype(np.int64))
+                last.append(int(s.tokens[-1]))
             pos_l.append(p)
             slots_l.append(table[p // PAGE] * PAGE + p % PAGE)
             qs.append(row0 + row)
@@ -785,15 +1027,15 @@ class LayeredRunner(RunnerBase):
             ht += list(range(nh))
             row += m
         T = row
-        lists = np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft + hs + ht, dtype=np.int64)
-        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + [lists]).astype(np.int32))
+        lists = np.asarray(qs + ql + ctx + ss + ws + wt + fs + ft + hs + ht + last, dtype=np.int64)
+        meta = torch.from_numpy(np.concatenate(ids_l + pos_l + slots_l + prev_l + [lists]).astype(np.int32))
         if self.device.type == "cuda":
             meta = meta.pin_memory().to(self.device, non_blocking=True)
             bt = bt.pin_memory().to(self.device, non_blocking=True)
         d, o = {}, 0
-        for name, k in (("ids", T), ("pos", T), ("slots", T), ("qs", n), ("ql", n), ("ctx", n), ("ss", n),
-                        ("ws", len(ws)), ("wt", len(ws)), ("fs", len(fs)), ("ft", len(fs)), ("hs", len(hs)),
-                        ("ht", len(hs))):
+        for name, k in (("ids", T), ("pos", T), ("slots", T), ("prev", T if self.bracket else 0), ("qs", n), ("ql", n),
+                        ("ctx", n), ("ss", n), ("ws", len(ws)), ("wt", len(ws)), ("fs", len(fs)), ("ft", len(fs)),
+                        ("hs", len(hs)), ("ht", len(hs)), ("last", len(last))):
             d[name], o = meta[o:o + k], o + k
         d["bt"] = bt
         d["qt"] = ATTN_ROWS_TILE
@@ -814,7 +1056,8 @@ class LayeredRunner(RunnerBase):
             return
         T, qs, ql, g = self._pack(seqs)
         d = self._buffers(T)
-        self._layers(T, d, g["ids"], g["pos"], g["slots"], [g], trace)
+        self._layers(T, d, g["ids"], g["pos"], g["slots"], [g], trace, prev=(g["prev"], None, None))
+        self._remember_last(seqs, g)
         self._prefill_sample(seqs, d["resid"], qs, ql, ring_row)
         self._keep_logits(seqs, d["resid"], qs)
 
@@ -831,7 +1074,9 @@ class LayeredRunner(RunnerBase):
         pos = torch.cat([self.positions[r], g["pos"]])
         slots = torch.cat([self.slots[r], g["slots"]])
         d = self._buffers(M)
-        self._layers(M, d, ids, pos, slots, [self._decode_group(B), g])
+        prev = (torch.cat([self.prev_ids[r], g["prev"]]), self.prev_ids[r], self.q_len[r]) if self.bracket else None
+        self._layers(M, d, ids, pos, slots, [self._decode_group(B), g], prev=prev)
+        self._remember_last(seqs, g)
         self._lm_head(d["resid"][r], self.logits[r])
         self._sample_commit(B)
         ops.ring_advance(self.ring_counter)

@@ -186,6 +186,7 @@ class PrefillSeq:
     block_table: list       # the sequence's full block table
     last_chunk: bool        # sample a token after this chunk
     want: tuple = ()        # offsets in this chunk whose logits the caller keeps (RunnerBase.kept_logits)
+    prev_token: int = -1    # the token before tokens[0] (start_pos > 0): embeddings that hash token pairs read it
 
 
 class RunnerBase:

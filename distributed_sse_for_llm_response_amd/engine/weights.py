@@ -260,6 +260,10 @@ class LayeredWeights:
     head_t: torch.Tensor = None  # the head in the tiled layout when its shape fits (head then None)
     step: torch.Tensor = None    # [passes, W] fp32: the vector added before each pass of a looped span (or None)
     ones: torch.Tensor = None    # [streams] fp32 ones of a design on several residual streams (or None)
+    bigram: torch.Tensor = None  # [buckets + 1, W] hashed (previous token, token) rows added to the embedding (or None)
+    side_embed: torch.Tensor = None  # [vocab, layers * dim] per-layer token inputs (or None)
+    loop_in: torch.Tensor = None     # [W, 2 W] projection of [stream | embedding output] that opens a loop pass
+    loop_in_t: torch.Tensor = None
 
     @property
     def vocab_local(self) -> int:
@@ -282,7 +286,8 @@ class LayeredWeights:
 
         for L in self.layers:
             n += size(L)
-        return n + sum(size(t) for t in (self.embed, self.final_norm, self.head, self.head_t, self.step, self.ones))
+        return n + sum(size(t) for t in (self.embed, self.final_norm, self.head, self.head_t, self.step, self.ones,
+                                         self.bigram, self.side_embed, self.loop_in, self.loop_in_t))
 
 
 TILED_MIN = 1024  # smallest N and K that go to the tiled-layout GEMMs
@@ -675,3 +680,175 @@ def load_dironex_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> Laye
     for f in sorted(Path(path).glob("*.safetensors")):
         tensors.update(load_file(str(f)))
     return convert_dironex(cfg, tensors, device=device, dtype=dtype)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Designs with bracketing norms, hashed bigram embeddings and per-layer token inputs (models/murulorn.py).  Projections
+# that read the same input are ONE weight, as for the other configuration-driven families; norm gains (stored around
+# zero in the checkpoint: 1 + w is formed here, in fp32), decay parameters, the decay's and the output gate's second
+# projections and the router are fp32 in both element types.  **Rotation layout**: the design rotates neighbouring
+# coordinates (2i, 2i + 1); the engine's norm / rotation / attention kernels pair coordinate i with i + dims / 2.  The
+# rows of the query and key projections (and their norm gains) are therefore permuted inside every head so that pair
+# i lands on (i, i + dims / 2) -- a scalar product is the same under a common permutation of both operands and the
+# whole-row RMS norm does not see the order -- and so are the rows of the value projection (whose per-head RMS norm
+# does not see the order either) together with the COLUMNS of the output projection, which reads the heads' outputs in
+# the values' order.
+@dataclass
+class RotatedValueAttentionWeights:
+    big: torch.Tensor        # rows [q (H D) | k (G D) | v (G V) | g (H) | zero rows] x W, heads in rotate-half order
+    n_big: int
+    q_norm: torch.Tensor     # [H D] fp32, in the same order
+    k_norm: torch.Tensor     # [G D] fp32
+    o: torch.Tensor          # [W, H V], columns in the values' order
+    big_t: torch.Tensor = None
+    o_t: torch.Tensor = None
+
+
+@dataclass
+class ChannelDeltaWeights:
+    big: torch.Tensor        # rows [q (G D) | k (G D) | v (H V) | b (H) | a1 (ra) | g1 (rg) | zero rows] x W
+    n_big: int
+    conv: torch.Tensor       # [2 G D + H V, taps] fp32: the taps of q | k | v
+    a_log: torch.Tensor      # [H] fp32
+    dt_bias: torch.Tensor    # [H D] fp32
+    a2: torch.Tensor         # [H D, ra] fp32 (its input is the fp32 output of a1)
+    g2: torch.Tensor         # [H V, rg] fp32
+    norm: torch.Tensor       # [V] fp32
+    o: torch.Tensor          # [W, H V]
+    big_t: torch.Tensor = None
+    o_t: torch.Tensor = None
+
+
+@dataclass
+class SquaredReluFfWeights:
+    up: torch.Tensor         # [F, W]
+    down: torch.Tensor       # [W, F]
+    up_t: torch.Tensor = None
+    down_t: torch.Tensor = None
+
+
+@dataclass
+class SoftmaxRoutedFfWeights:
+    router: torch.Tensor     # [E, W] fp32 in both element types (the router runs in true fp32 on the fp32 row)
+    up: torch.Tensor         # [E, F, W]
+    down: torch.Tensor       # [E, W, F]
+
+
+@dataclass
+class TokenSideWeights:
+    gate: torch.Tensor       # [dim, W]
+    proj: torch.Tensor       # [W, dim]
+    norm: torch.Tensor       # [W] fp32, a plain gain
+    col0: int                # the layer's first column of the side table
+
+
+@dataclass
+class BracketLayer:
+    norm1: torch.Tensor      # [W] fp32 gains (1 + stored) of the norm before the mixer ...
+    norm1b: torch.Tensor     # ... and after it
+    mix: object
+    norm2: torch.Tensor = None
+    norm2b: torch.Tensor = None
+    mlp: object = None
+    side: TokenSideWeights = None
+
+
+def half_from_pairs(width: int, dims: int) -> torch.Tensor:
+    """Index list that moves a neighbouring pair (2i, 2i + 1) of the first `dims` of `width` coordinates to
+    (i, i + dims / 2): new[j] = old[index[j]]; the coordinates from `dims` on keep their place."""
+    idx = torch.arange(width)
+    half = dims // 2
+    idx[:half] = torch.arange(0, dims, 2)
+    idx[half:dims] = torch.arange(1, dims, 2)
+    return idx
+
+
+@torch.no_grad()
+def convert_murulorn(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """Checkpoint tensors {name: tensor} (models/murulorn.py tensor_shapes) -> the engine's grouped layout in `dtype`."""
+    from ..models.murulorn import ANY, SquaredReluSpec, tensor_shapes
+
+    for name, shape in tensor_shapes(cfg).items():
+        if name not in tensors:
+            raise KeyError(f"checkpoint lacks tensor {name!r}")
+        got = tuple(tensors[name].shape)
+        if len(got) != len(shape) or any(s != ANY and s != g for s, g in zip(shape, got)):
+            raise ValueError(f"tensor {name!r} has shape {got}, the configuration says {shape}")
+
+    def t(name):
+        return tensors[name].to(device=device, dtype=dtype).contiguous()
+
+    def f(name):
+        return tensors[name].to(device=device, dtype=torch.float32).contiguous()
+
+    def gain(name):
+        return (1.0 + tensors[name].to(device=device, dtype=torch.float32)).contiguous()
+
+    def cat(*parts):
+        w = torch.cat(parts, dim=0)
+        if w.shape[0] >= TILED_MIN and w.shape[0] % 128:
+            w = torch.cat([w, w.new_zeros(128 - w.shape[0] % 128, w.shape[1])], dim=0)
+        return w.contiguous()
+
+    def heads_perm(n_heads: int, width: int, dims: int) -> torch.Tensor:
+        one = half_from_pairs(width, dims)
+        return (torch.arange(n_heads)[:, None] * width + one[None, :]).reshape(-1).to(device)
+
+    W = cfg.width
+    layers = []
+    for i, L in enumerate(cfg.layers):
+        p, m = f"l{i}.", L.mixer
+        if L.kind == "attention":
+            pq, pk = heads_perm(m.heads, m.dim, m.rot_dims), heads_perm(m.kv_heads, m.dim, m.rot_dims)
+            pv, po = heads_perm(m.kv_heads, m.vdim, m.vdim), heads_perm(m.heads, m.vdim, m.vdim)
+            big = cat(t(p + "mix.q")[pq], t(p + "mix.k")[pk], t(p + "mix.v")[pv], t(p + "mix.g"))
+            mix = RotatedValueAttentionWeights(big=big, n_big=big.shape[0], q_norm=f(p + "mix.q.norm")[pq].contiguous(),
+                                               k_norm=f(p + "mix.k.norm")[pk].contiguous(),
+                                               o=t(p + "mix.o")[:, po].contiguous())
+        else:
+            if tensors[p + "mix.a2"].shape[1] != tensors[p + "mix.a1"].shape[0] or \
+                    tensors[p + "mix.g2"].shape[1] != tensors[p + "mix.g1"].shape[0]:
+                raise ValueError(f"layer {i}: a low-rank pair disagrees on its inner width")
+            big = cat(t(p + "mix.q"), t(p + "mix.k"), t(p + "mix.v"), t(p + "mix.b"), t(p + "mix.a1"), t(p + "mix.g1"))
+            mix = ChannelDeltaWeights(big=big, n_big=big.shape[0],
+                                      conv=torch.cat([f(p + "mix.q.conv"), f(p + "mix.k.conv"),
+                                                      f(p + "mix.v.conv")]).contiguous(),
+                                      a_log=f(p + "mix.A_log"), dt_bias=f(p + "mix.dt_bias"), a2=f(p + "mix.a2"),
+                                      g2=f(p + "mix.g2"), norm=f(p + "mix.norm"), o=t(p + "mix.o"))
+        _tile_fields(mix, ("big", "o"))
+        layer = BracketLayer(norm1=gain(p + "norm1"), norm1b=gain(p + "norm1b"), mix=mix)
+        fs = L.mlp
+        if fs is not None:
+            layer.norm2, layer.norm2b = gain(p + "norm2"), gain(p + "norm2b")
+            if isinstance(fs, SquaredReluSpec):
+                layer.mlp = SquaredReluFfWeights(up=t(p + "mlp.up"), down=t(p + "mlp.down"))
+                _tile_fields(layer.mlp, ("up", "down"))
+            else:
+                stack = lambda leaf: torch.stack([t(f"{p}mlp.e{e}.{leaf}") for e in range(fs.experts)]).contiguous()  # noqa: E731
+                layer.mlp = SoftmaxRoutedFfWeights(router=f(p + "mlp.router"), up=stack("up"), down=stack("down"))
+        if cfg.side_dim:
+            layer.side = TokenSideWeights(gate=t(p + "side.gate"), proj=t(p + "side.proj"), norm=f(p + "side.norm"),
+                                          col0=i * cfg.side_dim)
+        layers.append(layer)
+    embed = t("embed")
+    out = LayeredWeights(cfg=cfg, embed=embed, layers=layers, final_norm=gain("final.norm"), head=embed, dtype=dtype)
+    if fits_tiled(embed):    # the head is the embedding table: the gather keeps the row-major copy
+        out.head_t, out.head = tile_weight(embed), None
+    out.bigram = t("bigram") if cfg.bigram else None
+    out.side_embed = t("side.embed") if cfg.side_dim else None
+    if cfg.loop_times > 0:
+        out.loop_in = t("loop.in")
+        _tile_fields(out, ("loop_in",))
+    return out
+
+
+def load_murulorn_dir(cfg, path: str, device="cpu", dtype=torch.bfloat16) -> LayeredWeights:
+    """``*.safetensors`` of a checkpoint directory -> the engine's layout (the loader executes nothing from them)."""
+    from pathlib import Path
+
+    from safetensors.torch import load_file
+
+    tensors = {}
+    for f in sorted(Path(path).glob("*.safetensors")):
+        tensors.update(load_file(str(f)))
+    return convert_murulorn(cfg, tensors, device=device, dtype=dtype)

@@ -132,13 +132,37 @@ def _dironex() -> Family:
                   (torch.bfloat16, torch.float32))
 
 
+def _murulorn() -> Family:
+    from . import murulorn as U
+
+    def random_weights(cfg, device, dtype, seed, tp_rank, tp_size):
+        from ..engine.weights import convert_murulorn
+
+        cfg.validate(tp_size)
+        return convert_murulorn(cfg, U.init_weights(cfg, seed=seed, device=device), device=device, dtype=dtype)
+
+    def load_dir(cfg, path, device, dtype, tp_rank, tp_size):
+        from ..engine.weights import load_murulorn_dir
+
+        cfg.validate(tp_size)
+        return load_murulorn_dir(cfg, path, device=device, dtype=dtype)
+
+    def runner():
+        from ..engine.layered_runner import LayeredRunner
+
+        return LayeredRunner
+
+    return Family("murulorn", ("Murulorn",), U.MurulornConfig.from_dict, dict(U.CONFIGS), random_weights, load_dir, runner,
+                  (torch.bfloat16, torch.float32))
+
+
 _FAMILIES = None
 
 
 def families() -> dict:
     global _FAMILIES
     if _FAMILIES is None:
-        _FAMILIES = {f.name: f for f in (_mistral(), _muderax(), _surodra(), _dironex())}
+        _FAMILIES = {f.name: f for f in (_mistral(), _muderax(), _surodra(), _dironex(), _murulorn())}
     return _FAMILIES
 
 
@@ -182,6 +206,6 @@ def cache_blocks_for_budget(cfg, budget_bytes: int, tp_size: int = 1, elem_bytes
     """Pages of the family's cache that fit `budget_bytes`."""
     from ..engine.kv_cache import PAGE, KVCache
 
-    if getattr(cfg, "family", "mistral") in ("muderax", "surodra", "dironex"):
+    if getattr(cfg, "family", "mistral") in ("muderax", "surodra", "dironex", "murulorn"):
         return max(1, budget_bytes // max(1, cfg.cache_bytes_per_token(elem_bytes) * PAGE))
     return KVCache.blocks_for_budget(budget_bytes, cfg.num_layers, cfg.num_kv_heads // tp_size)

@@ -187,22 +187,28 @@ def sink_flash_ok(dtype, dim: int, vdim: int) -> bool:
 
 
 def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile, sink, gate, out,
-                   window: int, scale: float, qt: int, vt=None, split: bool = False):
+                   window: int, scale: float, qt: int, vt=None, split: bool = False, softcap: float = 0.0, out_rope=None):
     """Causal softmax attention of q [T, H, D] over paged keys [pages, 32, G, D] and values [pages, 32, G, V] (grouped
     heads), scores and weights in fp32; sink [H] adds exp(sink) to each head's denominator, gate [T, H] multiplies the
     head's output by its sigmoid.  `qt` query rows per work item (work_seq, work_tile).  With vt (transposed value
     pages [pages, G, V, 32], sink_flash_ok shapes, qt = 16): the MFMA form; split (V <= 128) lets the four waves of a
-    workgroup share one (tile, head) and split its pages, for decode steps."""
+    workgroup share one (tile, head) and split its pages, for decode steps.  softcap > 0: scores
+    softcap * tanh(scale q.k / softcap).  out_rope ([positions, V / 2, 2] (cos, sin), rotate-half pairs over the whole
+    value width): each head's weighted sum is turned back by the query row's own position before the gate -- with
+    values that were rotated by THEIR positions when cached, a value enters the output rotated by the distance (the
+    MFMA form then needs V % 32 == 0)."""
     if _hip(q):
         torch.ops.dsse.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, work_seq, work_tile,
-                                      sink, gate, out, window, scale, qt, vt, split)
+                                      sink, gate, out, window, scale, qt, vt, split, softcap, out_rope)
     else:
-        lref.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt)
+        lref.sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt,
+                            softcap, out_rope)
 
 
 def gate_math(x, kind: int, p1=None, p2=None, c: float = 1.0):
     """In place on fp32 x [T, N] (a column slice is fine): 0: exp(-exp(p1) * softplus(x + p2)); 1: sigmoid(x);
-    2: sigmoid(x)^(1 / c)."""
+    2: sigmoid(x)^(1 / c).  p1 and p2 hold N numbers, or N / k of them: each then serves k neighbouring columns (one
+    rate per head beside one bias per head and channel)."""
     if _hip(x):
         torch.ops.dsse.gate_math(x, kind, p1, p2, c)
     else:
@@ -271,12 +277,12 @@ def matrix_scan_chunked(q, k, v, decay, state, q_start, q_len, ctx_len, state_sl
         lref.matrix_scan(q, k, v, decay, None, state, q_start, q_len, ctx_len, state_slot, out, q_scale)
 
 
-def gated_head_norm(o, w, gate, eps: float, out):
-    """out [T, H * V] (element type) = o / rms(o) per head * w (or no gain) * silu(gate)."""
+def gated_head_norm(o, w, gate, eps: float, out, kind: int = 0):
+    """out [T, H * V] (element type) = o / rms(o) per head * w (or no gain) * silu(gate); kind 1: * sigmoid(gate)."""
     if _hip(o):
-        torch.ops.dsse.gated_head_norm(o, w, gate, eps, out)
+        torch.ops.dsse.gated_head_norm(o, w, gate, eps, out, kind)
     else:
-        lref.gated_head_norm(o, w, gate, eps, out)
+        lref.gated_head_norm(o, w, gate, eps, out, kind)
 
 
 def rms_mix(ya, wa, yb, wb, eps: float, coef: float, out):
@@ -320,11 +326,49 @@ def act_rows(x, out, kind: int, params=None, gate=None):
         lref.act_rows(x, out, kind, params, gate)
 
 
-def moe_route(z, correction, topk_idx, topk_w, groups: int, keep: int, scale: float):
-    """Group-limited sigmoid routing from fp32 logits z [M, E]: choice scores sigmoid(z) + correction [E]; of `groups`
-    equal groups of neighbouring experts only the `keep` with the largest sum of their two best choice scores are
-    eligible; the top experts by choice score get the weights sigmoid(z) / (their sum + 1e-20) * scale."""
+def moe_route(z, correction, topk_idx, topk_w, groups: int, keep: int, scale: float, kind: int = 0):
+    """Group-limited routing from fp32 logits z [M, E].  kind 0 (sigmoid): choice scores sigmoid(z) + correction [E]; of
+    `groups` equal groups of neighbouring experts only the `keep` with the largest sum of their two best choice scores
+    are eligible; the top experts by choice score get the weights sigmoid(z) / (their sum + 1e-20) * scale.  kind 1
+    (softmax): scores softmax(z) over ALL experts (correction may be None), a group's score is its largest score, the
+    chosen experts' weights are their scores as they are, times scale."""
     if _hip(z):
-        torch.ops.dsse.moe_route(z, correction, topk_idx, topk_w, groups, keep, scale)
+        torch.ops.dsse.moe_route(z, correction, topk_idx, topk_w, groups, keep, scale, kind)
     else:
-        lref.moe_route(z, correction, topk_idx, topk_w, groups, keep, scale)
+        lref.moe_route(z, correction, topk_idx, topk_w, groups, keep, scale, kind)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Designs with bracketing norms, hashed bigram embeddings and per-layer token inputs.
+def embed_pair_rows(ids, prev, positions, embed, pair, mul_prev: int, mul_cur: int, buckets: int, resid, x0=None,
+                    prev_out=None, keep=None):
+    """resid (fp32) = embed[ids] + pair[row] with row = (prev * mul_prev + ids * mul_cur) mod buckets, or the table's
+    last row (`buckets`) at position 0; pair None: the plain embedding.  x0 (optional, element type, may be a column
+    slice of a wider buffer) receives the same rows.  prev_out (optional, int32 [B], may be `prev` itself): the first B
+    rows store their token there when keep[i] > 0 -- a decode slot's token becomes its next token's predecessor."""
+    if _hip(resid):
+        torch.ops.dsse.embed_pair_rows(ids, prev, positions, embed, pair, mul_prev, mul_cur, buckets, resid, x0, prev_out,
+                                       keep)
+    else:
+        lref.embed_pair_rows(ids, prev, positions, embed, pair, mul_prev, mul_cur, buckets, resid, x0, prev_out, keep)
+
+
+def add_norm_rows(y, nsum: int, g_add, resid, g_out, eps: float, out=None, out32=None):
+    """The stream's step between sublayers of a design that norms a sublayer's input AND its output, in one pass over
+    the row: y given ([M * nsum, W] fp32; a row's nsum consecutive parts are summed first, the grouped experts' slots):
+    resid += y / rms(y) * g_add; out given (element type or fp32; a column slice of a wider buffer is fine):
+    out = resid / rms(resid) * g_out, or the stream itself when g_out is None; out32 (fp32) receives that row unrounded
+    (what a router reads).  Gains are fp32 [W]."""
+    if _hip(resid):
+        torch.ops.dsse.add_norm_rows(y, nsum, g_add, resid, g_out, eps, out, out32)
+    else:
+        lref.add_norm_rows(y, nsum, g_add, resid, g_out, eps, out, out32)
+
+
+def token_gate_rows(x, ids, table, col0: int, out):
+    """out [M, F] (element type) = gelu_tanh(x) * table[ids, col0 : col0 + F]: a gate computed from the stream times a
+    slice of a per-token table.  x fp32 (a column slice is fine)."""
+    if _hip(x):
+        torch.ops.dsse.token_gate_rows(x, ids, table, col0, out)
+    else:
+        lref.token_gate_rows(x, ids, table, col0, out)

@@ -264,7 +264,9 @@ def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, sc
     elif norm_kind == 2:
         v = v / torch.sqrt(v.pow(2).sum(-1, keepdim=True) + eps)
     elif norm_kind == 3:
-        v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+        v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        if norm_w is not None:
+            v = v * norm_w.float()
     if rope is not None and rope.shape[1] > 0:
         pos = positions[:T].long().clamp(0, rope.shape[0] - 1)
         v = rotate_half_rows(v, rope[pos], 2 * rope.shape[1])
@@ -281,10 +283,13 @@ def norm_rope_rows(x, norm_w, positions, rope, out, out_rows, norm_kind, eps, sc
             out_t[good // PAGE, :, :, vt_position(good % PAGE)] = v[ok]
 
 
-def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt=None):
+def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sink, gate, out, window, scale, vt=None,
+                   softcap=0.0, out_rope=None):
     """Softmax attention over paged keys [pages, PAGE, G, D] and values [pages, PAGE, G, V] with grouped heads; the
     denominator also holds exp(sink[h]) when sink is given; the head's output is multiplied by sigmoid(gate[row, h])
-    when gate is given.  With vt the values come from the transposed pages [pages, G, V, PAGE]."""
+    when gate is given.  With vt the values come from the transposed pages [pages, G, V, PAGE].  softcap > 0: scores
+    softcap * tanh(. / softcap).  out_rope [positions, V / 2, 2]: the head's output is turned BACK by the query's
+    position (rotate-half pairs), undoing the rotation of a value rotated by that same position."""
     H = q.shape[1]
     G = kcache.shape[2]
     kf = kcache.view(-1, G, kcache.shape[3]).float()
@@ -304,6 +309,8 @@ def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sin
             if vt is not None:  # the same numbers from the transposed pages, so a wrong place shows
                 v = vt[rows // PAGE, :, :, vt_position(rows % PAGE)].float()[:, grp]
             sc = torch.einsum("hd,jhd->hj", q[r0 + i].float(), k) * scale
+            if softcap > 0:
+                sc = softcap * torch.tanh(sc / softcap)
             mx = sc.max(-1, keepdim=True).values
             if sink is not None:
                 mx = torch.maximum(mx, sink.float()[:, None])
@@ -312,6 +319,10 @@ def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sin
             if sink is not None:
                 den = den + torch.exp(sink.float()[:, None] - mx)
             o = torch.einsum("hj,jhv->hv", e / den, v)
+            if out_rope is not None:
+                cs = out_rope[min(pos, out_rope.shape[0] - 1)].float().clone()
+                cs[:, 1] = -cs[:, 1]
+                o = rotate_half_rows(o[None], cs[None], 2 * out_rope.shape[1])[0]
             if gate is not None:
                 o = o * torch.sigmoid(gate[r0 + i].float())[:, None]
             out[r0 + i] = o.to(out.dtype)
@@ -320,8 +331,11 @@ def sink_attention(q, kcache, vcache, block_tables, q_start, q_len, ctx_len, sin
 def gate_math(x, kind, p1, p2, c):
     """In place on fp32 x [T, N]: kind 0: exp(-exp(p1) * softplus(x + p2)) (p1, p2 [N]); 1: sigmoid(x);
     2: sigmoid(x)^(1 / c) as exp(logsigmoid(x) / c)."""
-    if kind == 0:
-        x.copy_(torch.exp(-torch.exp(p1.float()) * torch.nn.functional.softplus(x + p2.float())))
+    if kind == 0:  # p1, p2 may be shorter than a row: each entry then serves a run of neighbouring columns
+        N = x.shape[1]
+        a = p1.float().repeat_interleave(N // p1.numel())
+        b = p2.float().repeat_interleave(N // p2.numel())
+        x.copy_(torch.exp(-torch.exp(a) * torch.nn.functional.softplus(x + b)))
     elif kind == 1:
         x.copy_(torch.sigmoid(x))
     else:
@@ -354,13 +368,14 @@ def matrix_scan(q, k, v, decay, beta, state, q_start, q_len, ctx_len, state_slot
         state[slot] = S
 
 
-def gated_head_norm(o, w, gate, eps, out):
-    """out [T, H * V] = o / rms(o over V) * w (w [V] or None) * silu(gate [T, H * V])."""
+def gated_head_norm(o, w, gate, eps, out, kind=0):
+    """out [T, H * V] = o / rms(o over V) * w (w [V] or None) * silu(gate [T, H * V]) (kind 1: sigmoid(gate))."""
     T, H, V = o.shape
     n = o.float() / torch.sqrt(o.float().pow(2).mean(-1, keepdim=True) + eps)
     if w is not None:
         n = n * w.float()
-    out.copy_((n.reshape(T, H * V) * torch.nn.functional.silu(gate.float())).to(out.dtype))
+    g = torch.sigmoid(gate.float()) if kind == 1 else torch.nn.functional.silu(gate.float())
+    out.copy_((n.reshape(T, H * V) * g).to(out.dtype))
 
 
 def rms_mix(ya, wa, yb, wb, eps, coef, out):
@@ -413,21 +428,74 @@ def act_rows(x, out, kind, params, gate):
     out.copy_(z.to(out.dtype))
 
 
-def moe_route(z, correction, topk_idx, topk_w, groups, keep, scale):
-    """Router logits z [M, E] fp32 -> the `top` experts with the largest sigmoid(z) + correction among the experts of
+def moe_route(z, correction, topk_idx, topk_w, groups, keep, scale, kind=0):
+    """kind 1: scores softmax(z) over all experts, a group's score is its largest score, the weights are the chosen
+    scores as they are (times scale).  kind 0: router logits z [M, E] fp32 -> the `top` experts with the largest sigmoid(z) + correction among the experts of
     the `keep` best of `groups` equal groups of neighbours (a group's score: the sum of its two largest such values);
     weights: the chosen sigmoid(z) over their sum (+ 1e-20), times scale.  Ties go to the lower index."""
     M, E = z.shape
     top = topk_idx.shape[1]
-    s = torch.sigmoid(torch.nan_to_num(z.float(), nan=0.0))
-    choice = s + correction.float()
+    zz = torch.nan_to_num(z.float(), nan=0.0)
+    s = torch.softmax(zz, dim=-1) if kind == 1 else torch.sigmoid(zz)
+    choice = s + correction.float() if correction is not None else s.clone()
     if groups > 1:
         per = choice.view(M, groups, E // groups)
-        gscore = per.topk(min(2, E // groups), dim=-1).values.sum(-1)
+        gscore = per.max(-1).values if kind == 1 else per.topk(min(2, E // groups), dim=-1).values.sum(-1)
         order = torch.argsort(gscore, dim=-1, descending=True, stable=True)[:, :keep]
         allow = torch.zeros(M, groups, dtype=torch.bool).scatter_(1, order, True)
         choice = per.masked_fill(~allow[:, :, None], float("-inf")).reshape(M, E)
     idx = torch.argsort(choice, dim=-1, descending=True, stable=True)[:, :top]
     w = s.gather(1, idx)
     topk_idx.copy_(idx.to(torch.int32))
-    topk_w.copy_(w / (w.sum(-1, keepdim=True) + 1e-20) * scale)
+    topk_w.copy_(w * scale if kind == 1 else w / (w.sum(-1, keepdim=True) + 1e-20) * scale)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Designs with bracketing norms, hashed bigram embeddings and per-layer token inputs (models/murulorn.py)
+def embed_pair_rows(ids, prev, positions, embed, pair, mul_prev, mul_cur, buckets, resid, x0, prev_out, keep):
+    """resid (fp32) = embed[ids] + pair[row], row = (prev * mul_prev + ids * mul_cur) mod buckets, or `buckets` (the
+    table's last row) at position 0; x0 (optional, element type, may be a column slice) receives the same rows;
+    prev_out (optional, [B]): prev_out[i] = ids[i] for the first B rows whose keep[i] > 0 (decode slots remember their
+    token as the next one's predecessor)."""
+    M = resid.shape[0]
+    idx = ids[:M].long()
+    idx = torch.where((idx >= 0) & (idx < embed.shape[0]), idx, torch.zeros_like(idx))
+    rows = embed[idx].float()
+    if pair is not None:
+        pv = prev[:M].long().clamp(min=0)
+        r = (pv * mul_prev + idx * mul_cur) % buckets
+        r = torch.where(positions[:M].long() <= 0, torch.full_like(r, buckets), r)
+        rows = rows + pair[r].float()
+    if prev_out is not None:
+        B = prev_out.shape[0]
+        new = torch.where(keep[:B] > 0, ids[:B].to(prev_out.dtype), prev_out) if keep is not None else ids[:B]
+        prev_out.copy_(new)
+    resid.copy_(rows)
+    if x0 is not None:
+        x0.copy_(rows.to(x0.dtype))
+
+
+def add_norm_rows(y, nsum, g_add, resid, g_out, eps, out, out32):
+    """The residual stream's step of a design with a norm before AND after each sublayer.  y given ([M * nsum, W] fp32,
+    a row's nsum consecutive parts are summed first): resid += y / rms(y) * g_add.  out given (element type or fp32, may
+    be a column slice): out = resid / rms(resid) * g_out, or resid itself without g_out; out32 (optional, fp32) receives
+    the same row unrounded."""
+    if y is not None:
+        v = y.float().view(resid.shape[0], nsum, -1).sum(1)
+        resid.add_(v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * g_add.float())
+    if out is not None or out32 is not None:
+        n = resid
+        if g_out is not None:
+            n = resid / torch.sqrt(resid.pow(2).mean(-1, keepdim=True) + eps) * g_out.float()
+        if out is not None:
+            out.copy_(n.to(out.dtype))
+        if out32 is not None:
+            out32.copy_(n)
+
+
+def token_gate_rows(x, ids, table, col0, out):
+    """out [M, F] = gelu_tanh(x) * table[ids, col0 : col0 + F] for fp32 x (a column slice is fine)."""
+    F = x.shape[1]
+    idx = ids[:x.shape[0]].long()
+    idx = torch.where((idx >= 0) & (idx < table.shape[0]), idx, torch.zeros_like(idx))
+    out.copy_((gelu_tanh(x.float()) * table[idx, col0:col0 + F].float()).to(out.dtype))

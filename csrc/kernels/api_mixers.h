@@ -60,6 +60,9 @@ struct SinkAttnParams {
   int H, G, D, V, window, qt, ldg;
   float scale;
   int f32;
+  float softcap;         // > 0: score = softcap * tanh(scale q.k / softcap)
+  const float2* out_rope;  // [out_rope_len, V / 2] (cos, sin) or null: each head's sum is turned back by the row's own
+  int out_rope_len;        // position, rotate-half pairs (m, m + V / 2), before the gate
 };
 
 struct MatrixScanParams {
@@ -126,16 +129,53 @@ struct StreamMixParams {
   int h_f32;
 };
 
+// The embedding of a design that adds a hashed row per (previous token, token) pair.
+struct EmbedPairParams {
+  const int* ids;        // [M]
+  const int* prev;       // [M] previous token of each row (with pair)
+  const int* positions;  // [M]: position 0 takes row `buckets`
+  const void* embed;     // [vocab, W] element type
+  const void* pair;      // [buckets + 1, W] element type or null
+  int vocab, buckets;
+  long long mul_prev, mul_cur;
+  float* resid;          // [M, W] fp32
+  void* x0;              // rows ldx0 apart, element type, or null: the same row once more
+  int ldx0;
+  int* prev_out;         // [n_prev_out] or null: row i < n_prev_out stores its token when keep[i] > 0 (keep null: always)
+  const int* keep;
+  int n_prev_out;
+  int M, W, f32;
+};
+
+// The stream's step of a design with a norm before and after each sublayer.
+struct AddNormParams {
+  const float* y;        // [M * nsum, W] or null: resid += rms-norm(sum of the row's parts) * g_add
+  int nsum;
+  const float* g_add;    // [W]
+  float* resid;          // [M, W] fp32
+  const float* g_out;    // [W] or null: out = resid itself
+  void* out;             // rows ldo apart (fp32 when out_f32, else bf16) or null
+  float* out32;          // [M, W] fp32 copy of the unrounded output row, or null
+  int M, W, ldo, out_f32;
+  float eps;
+};
+
 }  // namespace dsse
 
 extern "C" {
+hipError_t dsse_embed_pair_rows(const dsse::EmbedPairParams* p, hipStream_t st);
+hipError_t dsse_add_norm_rows(const dsse::AddNormParams* p, hipStream_t st);
+// out [M, F] = gelu_tanh(x) * table[ids, col0 : col0 + F] (table rows ldt apart)
+hipError_t dsse_token_gate_rows(const float* x, int ldx, const int* ids, const void* table, int vocab, int ldt, int col0,
+                                void* out, int M, int F, int f32, hipStream_t st);
 hipError_t dsse_stream_mix(const dsse::StreamMixParams* p, hipStream_t st);
 // out [M, F] = act(x) * sigmoid(gate): kind 0 identity, 1 xIELU with params = (a_p, a_n), 2 relu^2; gate may be null
 hipError_t dsse_act_rows(const float* x, int ldx, void* out, int M, int F, int kind, const float* params,
                          const float* gate, int ldg, int f32, hipStream_t st);
-// group-limited sigmoid routing from fp32 logits [M, E] (E <= 256)
+// group-limited routing from fp32 logits [M, E] (E <= 256); kind 0: sigmoid scores + correction, groups by the sum of
+// their two best, weights renormalised; kind 1: softmax scores (corr may be null), groups by their best, weights as is
 hipError_t dsse_moe_route(const float* z, const float* corr, int M, int E, int top, int groups, int keep, float scale,
-                          int* topk_idx, float* topk_w, hipStream_t st);
+                          int kind, int* topk_idx, float* topk_w, hipStream_t st);
 hipError_t dsse_stream_step(const dsse::StreamStepParams* p, hipStream_t st);
 hipError_t dsse_gated_act(const float* gu, int ldg, void* h, int M, int F, int kind, int f32, hipStream_t st);
 hipError_t dsse_norm_rope_rows(const dsse::NormRopeParams* p, hipStream_t st);
@@ -144,12 +184,14 @@ hipError_t dsse_sink_attention(int num_work, const dsse::SinkAttnParams* p, hipS
 // transposed pages vt [pages, G, V, kBS] (keys permuted inside a page as the MFMA's k axis wants them)
 // split (V <= 128): the four waves of a workgroup share one (tile, head) and split its pages -- decode steps
 hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* p, const void* vt, int split, hipStream_t st);
-hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, const float* p2, float c,
-                          hipStream_t st);
+// p1 / p2 hold N / rep1 and N / rep2 numbers: entry j serves columns [j rep, (j + 1) rep)
+hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, int rep1, const float* p2, int rep2,
+                          float c, hipStream_t st);
 hipError_t dsse_matrix_scan(const dsse::MatrixScanParams* p, hipStream_t st);
 hipError_t dsse_scan_carry(const dsse::ScanCarryParams* p, hipStream_t st);
+// gate_kind 0: silu(gate), 1: sigmoid(gate)
 hipError_t dsse_gated_head_norm(const float* o, const float* w, const float* gate, int ldg, void* out, int M, int H,
-                                int V, float eps, int f32, hipStream_t st);
+                                int V, float eps, int gate_kind, int f32, hipStream_t st);
 hipError_t dsse_rms_mix(const float* ya, const float* wa, const float* yb, const float* wb, float* out, int M, int W,
                         float eps, float coef, hipStream_t st);
 hipError_t dsse_logit_cap(float* logits, long long n, float scale, float cap, hipStream_t st);

@@ -131,7 +131,7 @@ void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& posi
   TORCH_CHECK(kind >= 0 && kind <= 3 && p.D <= 512, "kind 0..3, head width <= 512");
   p.kind = (int)kind;
   p.norm_w = opt_f32(norm_w, "norm_w", kind == 3 ? (int64_t)p.D : (int64_t)p.nh * p.D);
-  TORCH_CHECK((kind != 1 && kind != 3) || p.norm_w, "kinds 1 and 3 need norm_w");
+  TORCH_CHECK(kind != 1 || p.norm_w, "kind 1 needs norm_w");
   if (rope.has_value() && rope->numel() > 0) {
     f32t(*rope, "rope");
     i32(positions, "positions");
@@ -176,7 +176,7 @@ void norm_rope_rows(const Tensor& x, const OptTensor& norm_w, const Tensor& posi
 void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache, const Tensor& block_tables,
                     const Tensor& q_start, const Tensor& q_len, const Tensor& ctx_len, const Tensor& work_seq,
                     const Tensor& work_tile, const OptTensor& sink, const OptTensor& gate, Tensor& out, int64_t window,
-                    double scale, int64_t qt, const OptTensor& vt, bool split) {
+                    double scale, int64_t qt, const OptTensor& vt, bool split, double softcap, const OptTensor& out_rope) {
   f32t(q, "q");
   gpu(kcache, "kcache");
   gpu(vcache, "vcache");
@@ -222,6 +222,16 @@ void sink_attention(const Tensor& q, const Tensor& kcache, const Tensor& vcache,
   p.window = (int)std::min<int64_t>(window, INT_MAX), p.qt = (int)qt;
   p.scale = (float)scale;
   p.f32 = elem(kcache, "kcache");
+  TORCH_CHECK(softcap >= 0, "softcap >= 0");
+  p.softcap = (float)softcap;
+  if (out_rope.has_value()) {
+    f32t(*out_rope, "out_rope");
+    TORCH_CHECK(out_rope->dim() == 3 && out_rope->size(2) == 2 && 2 * out_rope->size(1) == p.V && out_rope->size(0) >= 1,
+                "out_rope must be [P, V / 2, 2]");
+    TORCH_CHECK(!vt.has_value() || p.V % 32 == 0, "the MFMA form turns outputs back only for V % 32 == 0");
+    p.out_rope = reinterpret_cast<const float2*>(out_rope->data_ptr<float>());
+    p.out_rope_len = (int)out_rope->size(0);
+  }
   if (vt.has_value()) {  // MFMA form: work_tile counts tiles of 16 rows
     gpu(*vt, "vt");
     TORCH_CHECK(kcache.scalar_type() == at::kBFloat16 && vt->scalar_type() == at::kBFloat16, "the MFMA form is bf16");
@@ -240,11 +250,15 @@ void gate_math(Tensor& x, int64_t kind, const OptTensor& p1, const OptTensor& p2
   col_view(x, "x");
   const int M = (int)x.size(0), N = (int)x.size(1);
   TORCH_CHECK(kind >= 0 && kind <= 2, "kind 0..2");
-  const float* a = opt_f32(p1, "p1", N);
-  const float* b = opt_f32(p2, "p2", N);
+  // p1 / p2 hold one number per column, or one per run of neighbouring columns
+  const int64_t n1 = p1.has_value() ? p1->numel() : N, n2 = p2.has_value() ? p2->numel() : N;
+  TORCH_CHECK(n1 >= 1 && n2 >= 1 && N % n1 == 0 && N % n2 == 0, "p1 and p2 must divide the row into equal runs");
+  const float* a = opt_f32(p1, "p1", n1);
+  const float* b = opt_f32(p2, "p2", n2);
   TORCH_CHECK(kind != 0 || (a && b), "kind 0 needs p1 and p2");
   TORCH_CHECK(kind != 2 || c > 0, "kind 2 needs c > 0");
-  DSSE_CHECK_HIP(dsse_gate_math(x.data_ptr<float>(), (int)x.stride(0), M, N, (int)kind, a, b, (float)c, cur_stream()));
+  DSSE_CHECK_HIP(dsse_gate_math(x.data_ptr<float>(), (int)x.stride(0), M, N, (int)kind, a, (int)(N / n1), b, (int)(N / n2),
+                                (float)c, cur_stream()));
 }
 
 void matrix_scan(const Tensor& q, const Tensor& k, const Tensor& v, const OptTensor& decay, const OptTensor& beta,
@@ -395,7 +409,7 @@ void matrix_scan_chunked(const Tensor& q, const Tensor& k, const Tensor& v, cons
   DSSE_CHECK_HIP(dsse_matrix_scan(&p, cur_stream()));
 }
 
-void gated_head_norm(const Tensor& o, const OptTensor& w, const Tensor& gate, double eps, Tensor& out) {
+void gated_head_norm(const Tensor& o, const OptTensor& w, const Tensor& gate, double eps, Tensor& out, int64_t kind) {
   f32t(o, "o");
   col_view(gate, "gate");
   gpu(out, "out");
@@ -404,7 +418,7 @@ void gated_head_norm(const Tensor& o, const OptTensor& w, const Tensor& gate, do
   TORCH_CHECK(gate.size(0) == M && gate.size(1) == (int64_t)H * V && out.size(0) == M && out.size(1) == (int64_t)H * V,
               "gate and out must be [T, H V]");
   DSSE_CHECK_HIP(dsse_gated_head_norm(o.data_ptr<float>(), opt_f32(w, "w", V), gate.data_ptr<float>(),
-                                      (int)gate.stride(0), out.data_ptr(), M, H, V, (float)eps, elem(out, "out"),
+                                      (int)gate.stride(0), out.data_ptr(), M, H, V, (float)eps, (int)kind, elem(out, "out"),
                                       cur_stream()));
 }
 
@@ -506,28 +520,134 @@ void act_rows(const Tensor& x, Tensor& out, int64_t kind, const OptTensor& param
                                (int)kind, pp, g, ldg, elem(out, "out"), cur_stream()));
 }
 
-void moe_route(const Tensor& z, const Tensor& correction, Tensor& topk_idx, Tensor& topk_w, int64_t groups, int64_t keep,
-               double scale) {
+void moe_route(const Tensor& z, const OptTensor& correction, Tensor& topk_idx, Tensor& topk_w, int64_t groups,
+               int64_t keep, double scale, int64_t kind) {
   f32t(z, "z");
-  f32t(correction, "correction");
+  TORCH_CHECK(kind == 0 || kind == 1, "kind: 0 sigmoid scores, 1 softmax scores");
+  TORCH_CHECK(kind == 1 || correction.has_value(), "sigmoid routing needs its correction");
   i32(topk_idx, "topk_idx");
   f32t(topk_w, "topk_w");
   TORCH_CHECK(z.dim() == 2 && topk_idx.dim() == 2, "z must be [M, E], topk_idx [M, top]");
   const int M = (int)z.size(0), E = (int)z.size(1), top = (int)topk_idx.size(1);
-  TORCH_CHECK(topk_idx.size(0) == M && topk_w.sizes() == topk_idx.sizes() && correction.numel() == E, "routing shapes");
+  TORCH_CHECK(topk_idx.size(0) == M && topk_w.sizes() == topk_idx.sizes(), "routing shapes");
+  const float* corr = opt_f32(correction, "correction", E);
   TORCH_CHECK(E >= 1 && E <= 256 && groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 &&
                   top <= keep * (E / groups),
               "routing: E <= 256, equal groups, 1 <= keep <= groups, top <= experts of the kept groups");
-  DSSE_CHECK_HIP(dsse_moe_route(z.data_ptr<float>(), correction.data_ptr<float>(), M, E, top, (int)groups, (int)keep,
-                                (float)scale, topk_idx.data_ptr<int>(), topk_w.data_ptr<float>(), cur_stream()));
+  DSSE_CHECK_HIP(dsse_moe_route(z.data_ptr<float>(), corr, M, E, top, (int)groups, (int)keep, (float)scale, (int)kind,
+                                topk_idx.data_ptr<int>(), topk_w.data_ptr<float>(), cur_stream()));
+}
+
+void embed_pair_rows(const Tensor& ids, const OptTensor& prev, const Tensor& positions, const Tensor& embed,
+                     const OptTensor& pair, int64_t mul_prev, int64_t mul_cur, int64_t buckets, Tensor& resid,
+                     const OptTensor& x0, const OptTensor& prev_out, const OptTensor& keep) {
+  f32t(resid, "resid");
+  gpu(embed, "embed");
+  i32(ids, "ids");
+  TORCH_CHECK(resid.dim() == 2 && embed.dim() == 2 && embed.size(1) == resid.size(1), "resid [M, W], embed [vocab, W]");
+  dsse::EmbedPairParams p{};
+  p.M = (int)resid.size(0), p.W = (int)resid.size(1);
+  p.f32 = elem(embed, "embed");
+  TORCH_CHECK(ids.numel() >= p.M, "ids too short");
+  p.ids = ids.data_ptr<int>();
+  p.embed = embed.data_ptr();
+  p.vocab = (int)embed.size(0);
+  if (pair.has_value()) {
+    gpu(*pair, "pair");
+    TORCH_CHECK(prev.has_value(), "the pair table needs each row's previous token");
+    i32(*prev, "prev");
+    i32(positions, "positions");
+    TORCH_CHECK(pair->scalar_type() == embed.scalar_type() && pair->dim() == 2 && pair->size(1) == p.W && buckets >= 1 &&
+                    pair->size(0) == buckets + 1,
+                "pair must be [buckets + 1, W] in embed's type");
+    TORCH_CHECK(prev->numel() >= p.M && positions.numel() >= p.M && mul_prev >= 0 && mul_cur >= 0, "prev / positions too short");
+    p.pair = pair->data_ptr();
+    p.prev = prev->data_ptr<int>();
+    p.positions = positions.data_ptr<int>();
+  }
+  p.buckets = (int)buckets, p.mul_prev = mul_prev, p.mul_cur = mul_cur;
+  p.resid = resid.data_ptr<float>();
+  if (x0.has_value()) {
+    gpu(*x0, "x0", false);
+    TORCH_CHECK(x0->scalar_type() == embed.scalar_type() && x0->dim() == 2 && x0->size(0) == p.M && x0->size(1) == p.W &&
+                    (p.W == 1 || x0->stride(1) == 1) && x0->stride(0) >= p.W,
+                "x0 must be [M, W] in embed's type with unit column stride");
+    p.x0 = x0->data_ptr();
+    p.ldx0 = (int)x0->stride(0);
+  }
+  if (prev_out.has_value()) {
+    i32(*prev_out, "prev_out");
+    p.prev_out = prev_out->data_ptr<int>();
+    p.n_prev_out = (int)std::min<int64_t>(prev_out->numel(), p.M);
+    if (keep.has_value()) {
+      i32(*keep, "keep");
+      TORCH_CHECK(keep->numel() >= p.n_prev_out, "keep too short");
+      p.keep = keep->data_ptr<int>();
+    }
+  }
+  DSSE_CHECK_HIP(dsse_embed_pair_rows(&p, cur_stream()));
+}
+
+void add_norm_rows(const OptTensor& y, int64_t nsum, const OptTensor& g_add, Tensor& resid, const OptTensor& g_out,
+                   double eps, const OptTensor& out, const OptTensor& out32) {
+  f32t(resid, "resid");
+  TORCH_CHECK(resid.dim() == 2 && nsum >= 1, "resid [M, W], nsum >= 1");
+  dsse::AddNormParams p{};
+  p.M = (int)resid.size(0), p.W = (int)resid.size(1);
+  p.resid = resid.data_ptr<float>();
+  p.nsum = (int)nsum;
+  if (y.has_value()) {
+    f32t(*y, "y");
+    TORCH_CHECK(y->numel() == (int64_t)p.M * nsum * p.W, "y must hold M * nsum rows of W");
+    TORCH_CHECK(g_add.has_value(), "y needs its norm's gain");
+    p.y = y->data_ptr<float>();
+    p.g_add = opt_f32(g_add, "g_add", p.W);
+  }
+  p.g_out = opt_f32(g_out, "g_out", p.W);
+  if (out.has_value()) {
+    gpu(*out, "out", false);
+    TORCH_CHECK(out->dim() == 2 && out->size(0) == p.M && out->size(1) == p.W && (p.W == 1 || out->stride(1) == 1) &&
+                    out->stride(0) >= p.W,
+                "out must be [M, W] with unit column stride");
+    p.out_f32 = elem(*out, "out");
+    p.out = out->data_ptr();
+    p.ldo = (int)out->stride(0);
+  }
+  if (out32.has_value()) {
+    f32t(*out32, "out32");
+    TORCH_CHECK(out32->numel() == (int64_t)p.M * p.W, "out32 must be [M, W]");
+    p.out32 = out32->data_ptr<float>();
+  }
+  p.eps = (float)eps;
+  DSSE_CHECK_HIP(dsse_add_norm_rows(&p, cur_stream()));
+}
+
+void token_gate_rows(const Tensor& x, const Tensor& ids, const Tensor& table, int64_t col0, Tensor& out) {
+  col_view(x, "x");
+  i32(ids, "ids");
+  gpu(table, "table");
+  gpu(out, "out");
+  const int M = (int)x.size(0), F = (int)x.size(1);
+  TORCH_CHECK(table.dim() == 2 && col0 >= 0 && col0 + F <= table.size(1), "table [vocab, columns] must hold col0 + F columns");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == M && out.size(1) == F && out.scalar_type() == table.scalar_type(),
+              "out must be [M, F] in the table's type");
+  TORCH_CHECK(ids.numel() >= M, "ids too short");
+  DSSE_CHECK_HIP(dsse_token_gate_rows(x.data_ptr<float>(), (int)x.stride(0), ids.data_ptr<int>(), table.data_ptr(),
+                                      (int)table.size(0), (int)table.size(1), (int)col0, out.data_ptr(), M, F,
+                                      elem(table, "table"), cur_stream()));
 }
 
 TORCH_LIBRARY_FRAGMENT(dsse, m) {
   m.def("stream_mix(Tensor? y, int nsum, float mult, Tensor(a!) streams, Tensor? ids, Tensor? embed, float embed_scale, "
         "Tensor? out_w, Tensor? mix, Tensor? in_w, Tensor? norm_w, float eps, Tensor(b!)? h, Tensor(c!)? total) -> ()");
   m.def("act_rows(Tensor x, Tensor(a!) out, int kind, Tensor? params=None, Tensor? gate=None) -> ()");
-  m.def("moe_route(Tensor z, Tensor correction, Tensor(a!) topk_idx, Tensor(b!) topk_w, int groups, int keep, "
-        "float scale) -> ()");
+  m.def("moe_route(Tensor z, Tensor? correction, Tensor(a!) topk_idx, Tensor(b!) topk_w, int groups, int keep, "
+        "float scale, int kind=0) -> ()");
+  m.def("embed_pair_rows(Tensor ids, Tensor? prev, Tensor positions, Tensor embed, Tensor? pair, int mul_prev, "
+        "int mul_cur, int buckets, Tensor(a!) resid, Tensor(b!)? x0, Tensor(c!)? prev_out, Tensor? keep) -> ()");
+  m.def("add_norm_rows(Tensor? y, int nsum, Tensor? g_add, Tensor(a!) resid, Tensor? g_out, float eps, "
+        "Tensor(b!)? out, Tensor(c!)? out32) -> ()");
+  m.def("token_gate_rows(Tensor x, Tensor ids, Tensor table, int col0, Tensor(a!) out) -> ()");
   m.def("stream_step(Tensor? y, float mult, Tensor(a!) resid, Tensor? ids, Tensor? embed, Tensor? vec, Tensor? alpha, "
         "Tensor? w, Tensor? b, Tensor(b!)? xb) -> ()");
   m.def("gated_act(Tensor gu, Tensor(a!) h, int kind=1) -> ()");
@@ -535,14 +655,14 @@ TORCH_LIBRARY_FRAGMENT(dsse, m) {
         "int kind, float eps, float scale=1.0, Tensor(b!)? out_t=None) -> ()");
   m.def("sink_attention(Tensor q, Tensor kcache, Tensor vcache, Tensor block_tables, Tensor q_start, Tensor q_len, "
         "Tensor ctx_len, Tensor work_seq, Tensor work_tile, Tensor? sink, Tensor? gate, Tensor(a!) out, int window, "
-        "float scale, int qt, Tensor? vt=None, bool split=False) -> ()");
+        "float scale, int qt, Tensor? vt=None, bool split=False, float softcap=0.0, Tensor? out_rope=None) -> ()");
   m.def("gate_math(Tensor(a!) x, int kind, Tensor? p1=None, Tensor? p2=None, float c=1.0) -> ()");
   m.def("matrix_scan(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor? beta, Tensor(a!) state, Tensor q_start, "
         "Tensor q_len, Tensor ctx_len, Tensor state_slot, Tensor(b!) out, float q_scale=1.0) -> ()");
   m.def("matrix_scan_chunked(Tensor q, Tensor k, Tensor v, Tensor? decay, Tensor(a!) state, Tensor q_len, Tensor ctx_len, "
         "Tensor state_slot, Tensor s_first, Tensor s_count, Tensor cmeta, Tensor(b!) scratch, Tensor(c!)? a_scratch, "
         "Tensor(d!) out, float q_scale=1.0) -> ()");
-  m.def("gated_head_norm(Tensor o, Tensor? w, Tensor gate, float eps, Tensor(a!) out) -> ()");
+  m.def("gated_head_norm(Tensor o, Tensor? w, Tensor gate, float eps, Tensor(a!) out, int kind=0) -> ()");
   m.def("rms_mix(Tensor ya, Tensor wa, Tensor yb, Tensor wb, float eps, float coef, Tensor(a!) out) -> ()");
   m.def("logit_cap(Tensor(a!) logits, float scale, float cap) -> ()");
 }
@@ -551,6 +671,9 @@ TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
   m.impl("stream_mix", &stream_mix);
   m.impl("act_rows", &act_rows);
   m.impl("moe_route", &moe_route);
+  m.impl("embed_pair_rows", &embed_pair_rows);
+  m.impl("add_norm_rows", &add_norm_rows);
+  m.impl("token_gate_rows", &token_gate_rows);
   m.impl("stream_step", &stream_step);
   m.impl("gated_act", &gated_act);
   m.impl("norm_rope_rows", &norm_rope_rows);

@@ -189,30 +189,43 @@ __global__ __launch_bounds__(256) void act_rows_kernel(const float* x, int ldx, 
 constexpr int kMaxRouteExperts = 256;
 
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr, int M,
-                                                       int E, int top, int groups, int keep, float scale, int* topk_idx,
-                                                       float* topk_w) {
+                                                       int E, int top, int groups, int keep, float scale, int kind,
+                                                       int* topk_idx, float* topk_w) {
   __shared__ float choice[kMaxRouteExperts], score[kMaxRouteExperts], gs[kMaxRouteExperts];
   const int row = blockIdx.x, lane = threadIdx.x;
   const float* zr = z + (int64_t)row * E;
   const float ninf = -__builtin_inff();
+  float zmax = ninf, zsum = 0.f;
+  if (kind == 1) {  // softmax over all experts: the row's maximum and the sum of exponentials, wave-wide
+    for (int e = lane; e < E; e += 64) {
+      const float v = zr[e];
+      zmax = fmaxf(zmax, v == v ? v : 0.0f);
+    }
+    zmax = wave_max(zmax);
+    for (int e = lane; e < E; e += 64) {
+      const float v = zr[e];
+      zsum += expf((v == v ? v : 0.0f) - zmax);
+    }
+    zsum = wave_sum(zsum);
+  }
   for (int e = lane; e < E; e += 64) {
     float v = zr[e];
     v = v == v ? v : 0.0f;
-    const float sg = 1.0f / (1.0f + expf(-v));
+    const float sg = kind == 1 ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
     score[e] = sg;
-    choice[e] = sg + corr[e];
+    choice[e] = corr ? sg + corr[e] : sg;
   }
   __syncthreads();
   if (groups > 1) {
     const int per = E / groups;
-    for (int o = lane; o < groups; o += 64) {  // a group's score: the sum of its two largest choice scores
+    for (int o = lane; o < groups; o += 64) {  // a group's score: the sum of its two largest choice scores (kind 1: the largest)
       float a = ninf, b = ninf;
       for (int j = 0; j < per; ++j) {
         const float c = choice[o * per + j];
         if (c > a) b = a, a = c;
         else if (c > b) b = c;
       }
-      gs[o] = per > 1 ? a + b : a;
+      gs[o] = per > 1 && kind == 0 ? a + b : a;
     }
     __syncthreads();
     // rank of a group = groups with a larger score (or the same score and a lower index); eligible when rank < keep
@@ -250,7 +263,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     }
     __syncthreads();
   }
-  const float inv = scale / (sum + 1e-20f);
+  const float inv = kind == 1 ? scale : scale / (sum + 1e-20f);
   __syncthreads();
   for (int k = lane; k < top; k += 64) topk_w[(int64_t)row * top + k] *= inv;
 }
@@ -316,10 +329,11 @@ extern "C" hipError_t dsse_act_rows(const float* x, int ldx, void* out, int M, i
 }
 
 extern "C" hipError_t dsse_moe_route(const float* z, const float* corr, int M, int E, int top, int groups, int keep,
-                                     float scale, int* topk_idx, float* topk_w, hipStream_t st) {
+                                     float scale, int kind, int* topk_idx, float* topk_w, hipStream_t st) {
   if (M <= 0) return hipSuccess;
   if (E > dsse::kMaxRouteExperts || groups < 1 || E % groups || top > E) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(dsse::moe_route_kernel, dim3(M), dim3(64), 0, st, z, corr, M, E, top, groups, keep, scale,
+  if ((kind != 0 && kind != 1) || (kind == 0 && !corr)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(dsse::moe_route_kernel, dim3(M), dim3(64), 0, st, z, corr, M, E, top, groups, keep, scale, kind,
                      topk_idx, topk_w);
   return hipGetLastError();
 }

@@ -4,6 +4,11 @@
 //   out     = sum_j exp(score_j - m) v_j / (sum_j exp(score_j - m) + exp(sink_h - m)),  m = max(max_j score_j, sink_h)
 //   out    *= sigmoid(gate[row, h])                                                      (optional)
 //
+// Options for designs that ask for them: capped scores, score_j = cap * tanh(scale (q . k_j) / cap); and an output
+// rotation -- every head's sum is turned back by the query row's own position over the whole value width (rotate-half
+// pairs (m, m + V / 2), angles from a (cos, sin) table), before the gate: with values that were rotated by THEIR
+// positions when they were cached, a value then enters the output rotated by its distance to the query.
+//
 // The sink is a learned logit with no key and no value: it only enlarges the denominator, so a head can attend to
 // "nothing".  Scores, the running maximum, the weights and the output sums are fp32 in both element types; queries
 // arrive in fp32 (normed and rotated), keys and values are read from their pages in the cache's element type.
@@ -85,8 +90,9 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnParams p) {
       page = (unsigned)page < (unsigned)p.num_blocks ? page : 0;
       const int krow = (page * kBS + j % kBS) * p.G + g;
       const float s_dot = dot_row(qs, kc + (int64_t)krow * D, D);
-      float s = s_dot;
-      s = on ? s * p.scale : -INFINITY;
+      float s = s_dot * p.scale;
+      if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
+      s = on ? s : -INFINITY;
       const float m_new = fmaxf(m, wave_max(s));  // finite: the chunk holds at least one key
       const float w = on ? expf(s - m_new) : 0.f;
       const float f = expf(m - m_new);            // 0 when m was -inf
@@ -122,9 +128,19 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnParams p) {
     }
     const float gate = p.gate ? 1.0f / (1.0f + expf(-p.gate[(int64_t)row * p.ldg + h])) : 1.0f;
     T* out = reinterpret_cast<T*>(p.out) + ((int64_t)row * p.H + h) * V;
+    const int half = V >> 1;
+    const float2* orp = p.out_rope ? p.out_rope + (int64_t)(pos < p.out_rope_len ? pos : p.out_rope_len - 1) * half : nullptr;
     for (int d = threadIdx.x; d < V; d += blockDim.x) {
       float o = 0.f;
       for (int w = 0; w < 4; ++w) o += acc_s[w][d] * fw[w];
+      if (orp) {  // back by the row's position: (a, b) -> (a cos + b sin, b cos - a sin)
+        const bool lo_half = d < half;
+        const int dp = lo_half ? d + half : d - half;
+        float op = 0.f;
+        for (int w = 0; w < 4; ++w) op += acc_s[w][dp] * fw[w];
+        const float2 c = orp[lo_half ? d : dp];
+        o = lo_half ? o * c.x + op * c.y : o * c.x - op * c.y;
+      }
       out[d] = (T)(o / den * gate);
     }
   }
@@ -227,7 +243,9 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
     for (int i = 0; i < 8; ++i) {
       const int key = pg * kBS + (i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4));
       const bool seen = c_ok && key <= c_pos && c_pos - key < p.window;
-      sv[i] = seen ? (i < 4 ? s0[i] : s1[i - 4]) * p.scale : -INFINITY;
+      float sc = (i < 4 ? s0[i] : s1[i - 4]) * p.scale;
+      if (p.softcap > 0.f) sc = p.softcap * tanhf(sc / p.softcap);
+      sv[i] = seen ? sc : -INFINITY;
       mx = fmaxf(mx, sv[i]);
     }
     mx = rows4_max(mx);
@@ -271,12 +289,21 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
       const int64_t row = q0 + tile * 16 + col;
       float mm = p.sink ? p.sink[h] : -INFINITY;
       for (int w = 0; w < 4; ++w) mm = fmaxf(mm, mg[(w * 16 + col) * ldm + V]);
-      float den = p.sink ? expf(p.sink[h] - mm) : 0.f, num = 0.f;
+      float den = p.sink ? expf(p.sink[h] - mm) : 0.f, num = 0.f, nump = 0.f;
+      const int half = V >> 1;
+      const bool lo_half = d < half;
+      const int dp = lo_half ? d + half : d - half;
       for (int w = 0; w < 4; ++w) {
         const float* src = mg + (w * 16 + col) * ldm;
         const float f = src[V] == -INFINITY ? 0.f : expf(src[V] - mm);
         den += src[V + 1] * f;
         num += src[d] * f;
+        nump += src[dp] * f;
+      }
+      if (p.out_rope) {  // back by the row's position
+        const int ps = pos0 + tile * 16 + col;
+        const float2 c = p.out_rope[(int64_t)(ps < p.out_rope_len ? ps : p.out_rope_len - 1) * half + (lo_half ? d : dp)];
+        num = lo_half ? num * c.x + nump * c.y : num * c.x - nump * c.y;
       }
       float o = den > 0.f ? num / den : 0.f;
       if (p.gate) o *= 1.0f / (1.0f + expf(-p.gate[row * p.ldg + h]));
@@ -294,6 +321,18 @@ __global__ __launch_bounds__(256) void sink_flash_kernel(SinkAttnParams p, const
     }
     float inv = den > 0.f ? f / den : 0.0f;
     if (p.gate) inv *= 1.0f / (1.0f + expf(-p.gate[c_row * p.ldg + h]));
+    if (p.out_rope) {  // NT is even (the host checks V % 32 == 0): dimension m = 16 n + 4 g + i pairs with tile n + NT / 2
+      const float2* orp = p.out_rope + (int64_t)(c_pos < p.out_rope_len ? c_pos : p.out_rope_len - 1) * (V >> 1);
+#pragma unroll
+      for (int n = 0; n < NT / 2; ++n)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float2 c = orp[16 * n + 4 * g + i];
+          const float a = O[n][i], b = O[n + NT / 2][i];
+          O[n][i] = a * c.x + b * c.y;
+          O[n + NT / 2][i] = b * c.x - a * c.y;
+        }
+    }
     bf16* out = reinterpret_cast<bf16*>(p.out) + (c_row * p.H + h) * V;
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
@@ -327,6 +366,7 @@ extern "C" hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* 
   if (num_work <= 0 || p->H <= 0) return hipSuccess;
   if (p->f32 || p->D % 32 || p->V % 16 || p->V > 512 || p->D > 512 || p->H % p->G) return hipErrorInvalidValue;
   if (split && p->V > 128) return hipErrorInvalidValue;  // the merge area has to fit 64 KB of LDS
+  if (p->out_rope && p->V % 32) return hipErrorInvalidValue;  // both halves of a rotation pair are whole 16-wide tiles
   const bf16* v = reinterpret_cast<const bf16*>(vt);
   switch (p->V / 16) {
 #define DSSE_FLASH_CASE(n) case n: dsse::launch_flash<n>(num_work, *p, v, split, st); break;
@@ -342,6 +382,7 @@ extern "C" hipError_t dsse_sink_flash(int num_work, const dsse::SinkAttnParams* 
 extern "C" hipError_t dsse_sink_attention(int num_work, const dsse::SinkAttnParams* p, hipStream_t st) {
   if (num_work <= 0 || p->H <= 0) return hipSuccess;
   if (p->D > 512 || p->V > dsse::kMaxV || p->H % p->G) return hipErrorInvalidValue;
+  if (p->out_rope && p->V % 2) return hipErrorInvalidValue;
   dim3 grid(num_work, p->H);
   if (p->f32) hipLaunchKernelGGL(dsse::sink_attention_kernel<float>, grid, dim3(256), 0, st, *p);
   else hipLaunchKernelGGL(dsse::sink_attention_kernel<bf16>, grid, dim3(256), 0, st, *p);

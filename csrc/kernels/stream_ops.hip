@@ -4,11 +4,11 @@
 //                    that needs no row statistic, so the add and the norm are one pass over the row)
 //   gated_act        h = act(gate) * up from the fused gate | up projection's fp32 output (SiLU or tanh-form gelu)
 //   norm_rope_rows   a row of heads: RMS norm over the whole row with a gain, a unit vector per head, an RMS norm per
-//                    head with one gain vector for all heads, or nothing;
+//                    head with one gain vector for all heads (or without a gain), or nothing;
 //                    rotate-half rotation of each head's leading coordinates; a scale; written to a chosen output row
 //                    (a cache row: keys and values go straight into their pages) in fp32 or bf16
 //   gate_math        decays and gates in place: exp(-exp(A) softplus(x + dt)), sigmoid(x), sigmoid(x)^(1/tau)
-//   gated_head_norm  out = o / rms(o) * w * silu(gate) per (row, head)
+//   gated_head_norm  out = o / rms(o) * w * silu(gate) per (row, head), or * sigmoid(gate)
 //   rms_mix          out = c * (rms-norm(ya) * wa + rms-norm(yb) * wb)
 //   logit_cap        logits * scale, then cap * tanh(. / cap)
 //
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(NormRopeParams p) {
     }
     if (on)
       for (int i = lane; i < p.D; i += 64)
-        s[i] = xh[i] * inv * (p.kind == 1 ? p.norm_w[h * p.D + i] : (p.kind == 3 ? p.norm_w[i] : 1.0f));
+        s[i] = xh[i] * inv * (p.kind == 1 ? p.norm_w[h * p.D + i] : (p.kind == 3 && p.norm_w ? p.norm_w[i] : 1.0f));
     __syncthreads();  // the strip is written before it is read
     if (on)
       for (int i = lane; i < p.D; i += 64) {
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256) void norm_rope_rows_kernel(NormRopeParams p) {
 }
 
 __global__ __launch_bounds__(256) void gate_math_kernel(float* x, int ld, int M, int N, int kind, const float* p1,
-                                                        const float* p2, float c) {
+                                                        int rep1, const float* p2, int rep2, float c) {
   const int64_t n = (int64_t)M * N;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t r = i / N;
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void gate_math_kernel(float* x, int ld, int M,
     const float v = *px;
     float o;
     if (kind == 0) {
-      o = expf(-expf(p1[col]) * softplus_f(v + p2[col]));
+      o = expf(-expf(p1[col / rep1]) * softplus_f(v + p2[col / rep2]));
     } else if (kind == 1) {
       o = sigmoid_f(v);
     } else {
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void gate_math_kernel(float* x, int ld, int M,
 
 template <typename T>
 __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* o, const float* w, const float* gate, int ldg,
-                                                              T* out, int M, int H, int V, float eps) {
+                                                              T* out, int M, int H, int V, float eps, int gate_kind) {
   const int lane = threadIdx.x & 63;
   const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (row, head)
   if (item >= (int64_t)M * H) return;
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) void gated_head_norm_kernel(const float* o, co
   float ss = 0.f;
   for (int i = lane; i < V; i += 64) ss += oh[i] * oh[i];
   const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
-  for (int i = lane; i < V; i += 64) dst[i] = (T)(oh[i] * inv * (w ? w[i] : 1.0f) * silu_f(g[i]));
+  for (int i = lane; i < V; i += 64) dst[i] = (T)(oh[i] * inv * (w ? w[i] : 1.0f) * (gate_kind == 1 ? sigmoid_f(g[i]) : silu_f(g[i])));
 }
 
 __global__ __launch_bounds__(256) void rms_mix_kernel(const float* ya, const float* wa, const float* yb, const float* wb,
@@ -229,24 +229,25 @@ extern "C" hipError_t dsse_norm_rope_rows(const dsse::NormRopeParams* p, hipStre
   return hipGetLastError();
 }
 
-extern "C" hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, const float* p2, float c,
-                                     hipStream_t st) {
+extern "C" hipError_t dsse_gate_math(float* x, int ld, int M, int N, int kind, const float* p1, int rep1, const float* p2,
+                                     int rep2, float c, hipStream_t st) {
   if (M <= 0 || N <= 0) return hipSuccess;
+  if (rep1 < 1 || rep2 < 1) return hipErrorInvalidValue;
   hipLaunchKernelGGL(dsse::gate_math_kernel, dim3(dsse::flat_blocks((int64_t)M * N)), dim3(256), 0, st, x, ld, M, N, kind,
-                     p1, p2, c);
+                     p1, rep1, p2, rep2, c);
   return hipGetLastError();
 }
 
 extern "C" hipError_t dsse_gated_head_norm(const float* o, const float* w, const float* gate, int ldg, void* out, int M,
-                                           int H, int V, float eps, int f32, hipStream_t st) {
+                                           int H, int V, float eps, int gate_kind, int f32, hipStream_t st) {
   if (M <= 0 || H <= 0) return hipSuccess;
   const int blocks = (int)(((int64_t)M * H + 3) / 4);
   if (f32)
     hipLaunchKernelGGL(dsse::gated_head_norm_kernel<float>, dim3(blocks), dim3(256), 0, st, o, w, gate, ldg,
-                       reinterpret_cast<float*>(out), M, H, V, eps);
+                       reinterpret_cast<float*>(out), M, H, V, eps, gate_kind);
   else
     hipLaunchKernelGGL(dsse::gated_head_norm_kernel<bf16>, dim3(blocks), dim3(256), 0, st, o, w, gate, ldg,
-                       reinterpret_cast<bf16*>(out), M, H, V, eps);
+                       reinterpret_cast<bf16*>(out), M, H, V, eps, gate_kind);
   return hipGetLastError();
 }
 

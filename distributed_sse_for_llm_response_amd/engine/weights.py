@@ -758,8 +758,9 @@ def half_from_pairs(width: int, dims: int) -> torch.Tensor:
     (i, i + dims / 2): new[j] = old[index[j]]; the coordinates from `dims` on keep their place."""
     idx = torch.arange(width)
     half = dims // 2
-    idx[:half] = torch.arange(0, dims, 2)
-    idx[half:dims] = torch.arange(1, dims, 2)
+    if half > 0:
+        idx[:half] = torch.arange(0, dims, 2)
+        idx[half:dims] = torch.arange(1, dims, 2)
     return idx
 
 

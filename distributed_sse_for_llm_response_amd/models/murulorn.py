@@ -145,8 +145,7 @@ class MurulornConfig:
                     window=int(mask.get("size", NO_WINDOW)))
             elif L["type"] == "channel_delta":
                 mixer = ChannelDeltaSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
-                                         dim=int(m["dim"]), vdim=int(m["vdim"]), conv=int(m["conv"]),
-                                         decay_rank=int(m.get("decay_rank", ANY)), gate_rank=int(m.get("gate_rank", ANY)))
+                                         dim=int(m["dim"]), vdim=int(m["vdim"]), conv=int(m["conv"]))
             else:
                 raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
             f = L.get("mlp")
@@ -298,10 +297,12 @@ def tensor_shapes(cfg: MurulornConfig) -> dict:
 
 
 @torch.no_grad()
-def init_weights(cfg: MurulornConfig, seed: int = 0, device="cpu", dtype=torch.bfloat16, rank: int = 16) -> dict:
+def init_weights(cfg: MurulornConfig, seed: int = 0, device="cpu", dtype=torch.bfloat16, rank=16) -> dict:
     """Random weights in the checkpoint's naming: projections ~ N(0, 1 / fan-in), stored gains near 0 (bracketing norms)
-    or near 1 (plain norms), decay parameters spread so that fast and slow heads and channels occur.  `rank` fills the
-    inner widths that the configuration leaves to the checkpoint."""
+    or near 1 (plain norms), decay parameters spread so that fast and slow heads and channels occur.  `rank` (one number,
+    or one for the decay's and one for the gate's pair) fills the inner widths that the configuration leaves to the
+    checkpoint."""
+    ranks = (rank, rank) if isinstance(rank, int) else tuple(rank)
     dev = torch.device(device)
     gdev = dev if dev.type == "cuda" else torch.device("cpu")
     g = torch.Generator(device=gdev).manual_seed(seed)
@@ -314,8 +315,8 @@ def init_weights(cfg: MurulornConfig, seed: int = 0, device="cpu", dtype=torch.b
         return torch.rand(tuple(shape), generator=g, device=gdev)
 
     for name, shape in tensor_shapes(cfg).items():
-        shape = tuple(rank if x == ANY else x for x in shape)
         leaf = name.rsplit(".", 1)[-1]
+        shape = tuple(ranks[leaf in ("g1", "g2")] if x == ANY else x for x in shape)
         if name in ("embed", "bigram", "side.embed"):
             t = randn(shape) * (1.0 if name == "embed" else 0.5)
         elif leaf in ("norm1", "norm2", "norm1b", "norm2b") or name == "final.norm":

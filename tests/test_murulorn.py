@@ -1,0 +1,688 @@
+"""Murulorn on the engine against the plain oracle (tests/murulorn_oracle.py).
+
+Every test builds its own small configuration and random weights, drives the engine through its own entry points
+(LLMEngine.force_step for given tokens, add_request + step for generation) and compares the logits with the oracle's
+whole-sequence forward in float64.  The same tests run on the CPU (PyTorch reference ops: scheduler, cache and state
+plumbing) and, marked ``gpu``, on the HIP kernels in fp32 (every row, tight tolerance) and bf16 (the bulk of the rows:
+a close router call flips under bf16 rounding in these tiny random models and moves single rows).
+"""
+from __future__ import annotations
+
+import copy
+import json
+
+import pytest
+import torch
+
+import murulorn_oracle as oracle
+from distributed_sse_for_llm_response_amd.engine.engine import LLMEngine, SamplingParams
+from distributed_sse_for_llm_response_amd.engine.model_runner import PrefillSeq
+from distributed_sse_for_llm_response_amd.engine.weights import convert_murulorn, half_from_pairs
+from distributed_sse_for_llm_response_amd.models import registry
+from distributed_sse_for_llm_response_amd.models.murulorn import MurulornConfig, init_weights, tensor_shapes
+
+GPU = pytest.param("cuda", marks=pytest.mark.gpu)
+DEVICES = ["cpu", GPU]
+VOCAB = 53
+
+
+def att(heads=4, kv_heads=2, dim=10, vdim=6, window=9, dims=4, base=300.0, scale=0.3, cap=4.0, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "rot": {"base": base, "dims": dims}}
+    if window:
+        m["mask"] = {"size": window}
+    if cap:
+        m["softcap"] = cap
+    return {"type": "attention", "mlp": mlp, "mixer": m}
+
+
+def cd(heads=4, kv_heads=2, dim=6, vdim=10, conv=3, mlp=None):
+    return {"type": "channel_delta", "mlp": mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}}
+
+
+def dense(n=20):
+    return {"kind": "dense", "ff": n}
+
+
+def moe(experts=6, top=2, ff=9, groups=3, keep=2):
+    r = {"experts": experts, "top": top}
+    if groups:
+        r["groups"] = {"count": groups, "keep": keep}
+    return {"kind": "moe", "expert": {"ff": ff}, "router": r}
+
+
+def config(layers, width=26, vocab=VOCAB, eps=3e-6, loop=None, bigram=(37, 5, 3), side=7):
+    d = {"architecture": "Murulorn", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": copy.deepcopy(layers)}
+    if bigram:
+        d["embedding"] = {"bigram": {"buckets": bigram[0], "mul_prev": bigram[1], "mul_cur": bigram[2]}}
+    if side:
+        d["token_side"] = {"dim": side}
+    if loop:
+        d["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return d
+
+
+HYBRID = config([att(mlp=dense()), cd(mlp=moe()), att(heads=2, kv_heads=2, dim=8, vdim=8, window=33, dims=8, cap=0, mlp=moe(top=3)),
+                 cd(heads=3, kv_heads=3, dim=8, vdim=4, conv=2, mlp=dense(11))], loop=(1, 3, 2))
+
+
+class Model:
+    """Configuration + random weights + an engine on `device` in `dtype`."""
+
+    def __init__(self, cfg_dict, device, dtype=torch.float32, seed=0, max_tokens=256, max_seqs=4, tweak=None, rank=(5, 3)):
+        self.cfg_dict = cfg_dict
+        self.cfg = MurulornConfig.from_dict(cfg_dict)
+        self.weights = init_weights(self.cfg, seed=seed, rank=rank)
+        if tweak:
+            tweak(self.weights)
+        self.device, self.dtype = torch.device(device), dtype
+        w = convert_murulorn(self.cfg, self.weights, device=self.device, dtype=dtype)
+        fam = registry.family_of(self.cfg)
+        assert fam.name == "murulorn"
+        self.runner = registry.make_runner(fam, w, num_blocks=-(-max_tokens // 32), max_batch=max_seqs,
+                                           max_model_len=max_tokens, max_prefill_tokens=max_tokens, device=self.device,
+                                           use_graphs=False)
+        self.engine = LLMEngine(self.runner, eos_id=-1)
+        self.engine.watermark = 0
+
+    def expect(self, tokens, cfg_dict=None, weights=None):
+        return oracle.forward(cfg_dict or self.cfg_dict, weights or self.weights, tokens).float()
+
+    def check(self, got, want, what=""):
+        """Row-wise: rms of the difference (mean taken off) over the rms of the expected logits.  fp32 judges every
+        row; bf16 judges nine rows in ten and the median."""
+        got, want = got.detach().float().cpu(), want.float()
+        assert got.shape == want.shape, (got.shape, want.shape)
+        assert torch.isfinite(got).all(), what
+        d = got - want
+        d = d - d.mean(-1, keepdim=True)
+        err = d.pow(2).mean(-1).sqrt() / (want - want.mean(-1, keepdim=True)).pow(2).mean(-1).sqrt().clamp_min(1e-6)
+        if self.dtype == torch.float32:
+            assert float(err.max()) < 2e-4, f"{what}: worst row {int(err.argmax())} error {float(err.max()):.3g}"
+        else:
+            assert float((err < 6e-2).float().mean()) >= 0.9 and float(err.median()) < 3e-2, \
+                f"{what}: median {float(err.median()):.3g}, {int((err >= 6e-2).sum())} of {err.numel()} rows off"
+
+    def run_cut(self, cid, tokens, cuts, end=True):
+        """Feed `tokens` in portions of the given sizes (the last size repeats), all logits wanted."""
+        out, at, k = [], 0, 0
+        while at < len(tokens):
+            n = min(cuts[min(k, len(cuts) - 1)], len(tokens) - at)
+            last = at + n == len(tokens)
+            out.append(self.engine.force_step([(cid, tokens[at:at + n], list(range(n)))], [cid] if last and end else []))
+            at, k = at + n, k + 1
+        return torch.cat(out)
+
+
+def toks(n, vocab=VOCAB, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def modes(device):
+    return [torch.float32] if device == "cpu" else [torch.float32, torch.bfloat16]
+
+
+def gap(a, b, rows=slice(None)):
+    """Median over rows of |a - b| rms relative to b's rms: how far a variant of the design is from the design."""
+    a, b = a[rows], b[rows]
+    return float(((a - b).pow(2).mean(-1).sqrt() / b.pow(2).mean(-1).sqrt().clamp_min(1e-6)).median())
+
+
+def gap_max(a, b, rows=slice(None)):
+    """The largest such difference over the rows: whether a variant changes ANY of them."""
+    a, b = a[rows], b[rows]
+    return float(((a - b).pow(2).mean(-1).sqrt() / b.pow(2).mean(-1).sqrt().clamp_min(1e-6)).max())
+
+
+def scaled(names_and_factors):
+    """A weight tweak: tensors whose name ends with a given suffix are multiplied by a factor."""
+    def tweak(w):
+        for k in w:
+            for suffix, f in names_and_factors:
+                if k.endswith(suffix):
+                    w[k] = (w[k].float() * f).to(w[k].dtype)
+    return tweak
+
+
+def changed(weights, fn):
+    """A copy of the weights with fn(name, tensor) -> tensor or None (unchanged) applied."""
+    out = {}
+    for k, v in weights.items():
+        r = fn(k, v)
+        out[k] = v if r is None else r
+    return out
+
+
+# ---------------------------------------------------------------------------------------------- mechanisms alone
+BARE = dict(bigram=None, side=0)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,cfgd", [
+    ("attention, grouped heads, part of each head rotates", config([att()], **BARE)),
+    ("attention, a key head per head, whole heads rotate, no window, no cap", config([att(heads=3, kv_heads=3, dim=8, dims=8, window=None, cap=0)], **BARE)),
+    ("attention, one key head, window of one, queries and keys do not rotate", config([att(heads=3, kv_heads=1, window=1, dims=0)], **BARE)),
+    ("attention, two-wide values", config([att(heads=2, kv_heads=1, dim=4, vdim=2, window=5)], **BARE)),
+    ("channel delta, shared query / key heads", config([cd()], **BARE)),
+    ("channel delta, a key head per head, one tap", config([cd(heads=3, kv_heads=3, conv=1)], **BARE)),
+    ("channel delta, one key head, five taps", config([cd(heads=4, kv_heads=1, dim=5, vdim=3, conv=5)], **BARE)),
+    ("dense feed-forward", config([att(heads=1, kv_heads=1, mlp=dense())], **BARE)),
+    ("routed experts in groups", config([cd(heads=1, kv_heads=1, mlp=moe())], **BARE)),
+    ("routed experts, no groups, one expert per token", config([att(mlp=moe(experts=5, top=1, groups=None))], **BARE)),
+    ("routed experts, groups of one, all kept", config([att(mlp=moe(experts=4, top=4, groups=4, keep=4))], **BARE)),
+    ("routed experts, one group kept", config([cd(mlp=moe(experts=8, top=2, groups=4, keep=1))], **BARE)),
+    ("pair embedding alone", config([att(mlp=dense())], bigram=(11, 7, 2), side=0)),
+    ("pair embedding with one bucket", config([cd()], bigram=(1, 1, 1), side=0)),
+    ("token inputs alone", config([att(mlp=dense()), cd()], bigram=None, side=3)),
+    ("one-wide token input", config([cd(mlp=moe())], bigram=None, side=1)),
+    ("a loop of one layer, three passes", config([att(), cd(mlp=moe()), att(mlp=dense())], loop=(1, 2, 3))),
+    ("a loop of everything, one pass", config([cd(), att(mlp=dense())], loop=(0, 2, 1))),
+    ("a loop that starts the model and ends it", config([att(mlp=moe()), cd(mlp=dense())], loop=(0, 2, 2))),
+])
+def test_mechanism_alone(device, name, cfgd):
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype)
+        t = toks(37, seed=1)
+        m.check(m.run_cut("a", t, [len(t)]), m.expect(t), name + ", whole")
+        m.check(m.run_cut("b", t, [9, 1]), m.expect(t), name + ", decoding")
+
+
+def test_each_op_against_its_oracle_function():
+    """The reference ops the CPU engine runs on, one mechanism at a time, against the oracle's functions."""
+    from distributed_sse_for_llm_response_amd import ops
+    g = torch.Generator().manual_seed(5)
+    # routing: softmax over all experts, groups ranked by their best score, weights as they are
+    z = torch.randn(40, 12, generator=g) * 2
+    r = {"experts": 12, "top": 3, "groups": {"count": 4, "keep": 2}}
+    idx, w = oracle.route(z.double(), r)
+    ti, tw = torch.zeros(40, 3, dtype=torch.int32), torch.zeros(40, 3)
+    ops.moe_route(z, None, ti, tw, 4, 2, 1.0, 1)
+    assert torch.equal(ti.long().sort(-1).values, idx.sort(-1).values)
+    assert torch.allclose(tw.gather(1, ti.long().argsort(-1)), w.float().gather(1, idx.argsort(-1)), atol=1e-6)
+    assert float(tw.sum(-1).max()) < 1.0 - 1e-3, "the weights are not renormalised"
+    assert not torch.equal(idx.sort(-1).values, oracle.route(z.double(), {**r, "groups": None})[0].sort(-1).values)
+    # the pair embedding's rows
+    cfgd = config([att()], bigram=(11, 7, 2), side=0)
+    wts = {"embed": torch.randn(VOCAB, 26, generator=g), "bigram": torch.randn(12, 26, generator=g)}
+    t = toks(9, seed=3)
+    want = oracle.embedding(cfgd, {k: v.double() for k, v in wts.items()}, torch.tensor(t))
+    resid, x0 = torch.zeros(9, 26), torch.zeros(9, 26)
+    ids = torch.tensor(t, dtype=torch.int32)
+    prev = torch.tensor([-1] + t[:-1], dtype=torch.int32)
+    ops.embed_pair_rows(ids, prev, torch.arange(9, dtype=torch.int32), wts["embed"], wts["bigram"], 7, 2, 11, resid, x0)
+    assert torch.allclose(resid, want.float(), atol=1e-6) and torch.equal(resid, x0)
+    assert not torch.allclose(want[0], (wts["embed"][t[0]] + wts["bigram"][(t[0] * 2) % 11]).double()), "row 0 is the last row"
+    # a mid-sequence portion: position decides, not the row index
+    ops.embed_pair_rows(ids[4:], prev[4:], torch.arange(4, 9, dtype=torch.int32), wts["embed"], wts["bigram"], 7, 2, 11,
+                        resid[:5], None)
+    assert torch.allclose(resid[:5], want[4:].float(), atol=1e-6)
+    # add + norm rows: parts summed, normed, added; then the stream normed
+    y, res = torch.randn(5, 2, 8, generator=g), torch.randn(5, 8, generator=g)
+    ga, go = torch.randn(8, generator=g), torch.randn(8, generator=g)
+    want_res = res.double() + oracle.rms(y.double().sum(1), 1e-5) * ga.double()
+    out, out32 = torch.zeros(5, 8, dtype=torch.bfloat16), torch.zeros(5, 8)
+    ops.add_norm_rows(y.view(10, 8), 2, ga, res, go, 1e-5, out, out32)
+    assert torch.allclose(res, want_res.float(), atol=1e-5)
+    assert torch.allclose(out32, (oracle.rms(want_res, 1e-5) * go.double()).float(), atol=1e-5)
+    assert torch.equal(out, out32.to(torch.bfloat16))
+    # the token input's gate
+    x = torch.randn(9, 3, generator=g)
+    table = torch.randn(VOCAB, 12, generator=g)
+    sh = torch.zeros(9, 3)
+    ops.token_gate_rows(x, ids, table, 6, sh)
+    assert torch.allclose(sh, (oracle.gelu_tanh(x.double()) * table[ids.long(), 6:9].double()).float(), atol=1e-6)
+
+
+def test_rotation_layout():
+    """Neighbouring pairs (2i, 2i + 1) of the first `dims` coordinates land on the kernels' pairs (i, i + dims / 2); the
+    engine's (cos, sin) table holds the design's frequencies."""
+    from distributed_sse_for_llm_response_amd.models.surodra import HalfRotarySpec
+    from distributed_sse_for_llm_response_amd.ops.layers_reference import rotate_half_rows
+
+    assert half_from_pairs(10, 6).tolist() == [0, 2, 4, 1, 3, 5, 6, 7, 8, 9]
+    g = torch.Generator().manual_seed(1)
+    v = torch.randn(7, 2, 10, generator=g, dtype=torch.float64)
+    pos = torch.tensor([0, 1, 2, 5, 9, 30, 31])
+    want = oracle.rotate_pairs(v, 1.0, 300.0, 6, pos)
+    perm = half_from_pairs(10, 6)
+    table = HalfRotarySpec(dims=6, base=300.0).table(40)
+    got = rotate_half_rows(v[..., perm].float(), table[pos], 6)
+    assert torch.allclose(got.double(), want[..., perm], atol=1e-5)
+    back = oracle.rotate_pairs(want, -1.0, 300.0, 6, pos)
+    assert torch.allclose(back, v, atol=1e-12)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_layer_trace(device):
+    """The engine's layer trace (the stream after every layer run) against the oracle's."""
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype)
+        t = toks(21, seed=2)
+        got, want = [], []
+        m.runner.prefill([PrefillSeq(slot=0, tokens=t, start_pos=0, block_table=[0], last_chunk=False)], 0, trace=got)
+        oracle.forward(HYBRID, m.weights, t, want)
+        assert len(got) == len(want) == 6
+        tol = 1e-4 if dtype == torch.float32 else 3e-2
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert float((a.cpu().double() - b).abs().max() / b.abs().max()) < tol, f"layer run {i}"
+
+
+# ---------------------------------------------------------------------------------------------- cuts, batches, pools
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefill_against_token_by_token(device):
+    t = toks(45, seed=3)
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype)
+        want = m.expect(t)
+        whole = m.run_cut("w", t, [len(t)])
+        single = m.run_cut("s", t, [1])
+        m.check(whole, want, "whole prompt")
+        m.check(single, want, "token by token")
+        if dtype == torch.float32:
+            m.check(single, whole.cpu(), "token by token against the whole prompt")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[2], [3, 2, 7], [5, 1, 1, 2, 11], [31, 2, 1], [33, 1], [64, 2]])
+def test_portions(device, cuts):
+    """Portions cut inside pages, windows and the convolution's reach, down to two tokens."""
+    t = toks(70, seed=4)
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype)
+        m.check(m.run_cut("p", t, cuts), m.expect(t), f"portions {cuts}")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_unequal_batch_against_each_alone(device):
+    """Four requests of unequal length in one batch: portions of some beside single tokens of others, one sits out
+    steps, one ends early and its slot and pages go to a newcomer."""
+    seqs = {"a": toks(50, seed=5), "b": toks(9, seed=6), "c": toks(34, seed=7), "d": toks(1, seed=8), "e": toks(40, seed=9)}
+    plan = [{"a": 7, "b": 2, "c": 20}, {"a": 1, "b": 1, "d": 1}, {"a": 1, "c": 2, "b": 1}, {"a": 30, "b": 1, "e": 3},
+            {"a": 1, "b": 1, "c": 1, "e": 33}, {"a": 1, "b": 1, "c": 11, "e": 1}, {"a": 9, "b": 2, "e": 3}]
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype, max_tokens=256)
+        at = {k: 0 for k in seqs}
+        got = {k: [] for k in seqs}
+        for step in plan:
+            entries, end = [], []
+            for k, n in step.items():
+                n = min(n, len(seqs[k]) - at[k])
+                entries.append((k, seqs[k][at[k]:at[k] + n], list(range(n))))
+                at[k] += n
+                if at[k] == len(seqs[k]):
+                    end.append(k)
+            out = m.engine.force_step(entries, end)
+            o = 0
+            for k, tk, _ in entries:
+                got[k].append(out[o:o + len(tk)])
+                o += len(tk)
+        for k, t in seqs.items():
+            assert at[k] == len(t), k
+            m.check(torch.cat(got[k]), m.expect(t), f"request {k} in the batch")
+        assert m.engine.alloc.num_free == m.engine.alloc.num_blocks
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_pages_and_slots_used_again(device):
+    """A pool of three pages and two slots: every later request runs in pages and slots that held another one (its
+    keys and rotated values, its matrix states, convolution tails and previous token), in prompts and in decoding."""
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype, max_tokens=96, max_seqs=2)
+        for i, (n, cuts) in enumerate([(60, [60]), (64, [33, 1]), (40, [2, 30, 1]), (64, [64]), (5, [1])]):
+            t = toks(n, seed=30 + i)
+            keep = toks(20, seed=40 + i)
+            first = m.engine.force_step([(f"k{i}", keep[:10], list(range(10)))])
+            got = m.run_cut(f"r{i}", t, cuts)
+            rest = m.engine.force_step([(f"k{i}", keep[10:], list(range(10)))], [f"k{i}"])
+            m.check(got, m.expect(t), f"request {i}")
+            m.check(torch.cat([first, rest]), m.expect(keep), f"neighbour of request {i}")
+        assert m.engine.alloc.num_free == m.engine.alloc.num_blocks
+    m.engine.force_step([("held", toks(64, seed=1), [])])
+    with pytest.raises(MemoryError):
+        m.engine.force_step([("late", toks(64, seed=2), [])])
+
+
+# ---------------------------------------------------------------------------------------------- state that must not be lost
+@pytest.mark.parametrize("device", DEVICES)
+def test_previous_token_is_sequence_state(device):
+    """The pair embedding made large: a wrong predecessor at the start of a portion, after a decoded token, after a
+    step that the request sat out, or in a slot that another request used would move the logits.  The oracle with the
+    pairs hashed the other way round, or with position 0 treated like any other, is far away."""
+    cfgd = config([att(mlp=dense()), cd()], bigram=(41, 9, 4), side=0)
+    big = scaled([("bigram", 4.0)])
+    t, other = toks(40, seed=10), toks(12, seed=11)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, max_seqs=2, tweak=big)
+        want = m.expect(t)
+        swapped = copy.deepcopy(cfgd)
+        swapped["embedding"]["bigram"].update(mul_prev=4, mul_cur=9)
+        assert gap(m.expect(t, swapped), want) > 5e-2
+        first_like_rest = changed(m.weights, lambda k, v: torch.cat([v[:-1], v[:1]]) if k == "bigram" else None)
+        assert gap_max(m.expect(t, weights=first_like_rest), want) > 5e-2
+        m.run_cut("warm", other, [12])
+        m.check(m.run_cut("p", t, [3, 1, 1, 2, 1, 7, 1]), want, "portions and single tokens in turn")
+        # the request sits out steps while another one runs in the neighbouring slot
+        got = [m.engine.force_step([("s", t[:5], list(range(5)))])]
+        m.engine.force_step([("o", other[:6], [])])
+        got.append(m.engine.force_step([("s", t[5:6], [0]), ("o", other[6:7], [])]))
+        m.engine.force_step([("o", other[7:], [])], ["o"])
+        got.append(m.engine.force_step([("s", t[6:], list(range(len(t) - 6)))], ["s"]))
+        m.check(torch.cat(got), want, "a request that sat out steps")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slow_state_survives(device):
+    """Decays close to one and a write strength near one: what a channel-delta layer wrote 200 tokens ago still counts,
+    across portions, decoding and a slot that changes hands.  The oracle that forgets faster is far away."""
+    cfgd = config([cd(heads=2, kv_heads=1, dim=8, vdim=6, conv=2)], bigram=None, side=0)
+
+    def slow(w):
+        for k in w:
+            if k.endswith("A_log"):
+                w[k] = torch.full_like(w[k], -6.0)
+            if k.endswith("mix.b"):
+                w[k] = (w[k].float() * 3).to(w[k].dtype)
+
+    t = toks(230, seed=12)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, max_seqs=1, tweak=slow)
+        want = m.expect(t)
+        fast = changed(m.weights, lambda k, v: torch.full_like(v, 0.5) if k.endswith("A_log") else None)
+        assert gap(m.expect(t, weights=fast), want, slice(200, None)) > 5e-2
+        m.run_cut("warm", toks(50, seed=13), [50])
+        m.check(m.run_cut("a", t, [100, 2, 64, 1]), want, "portions, then decoding")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_decay_is_per_head_and_channel(device):
+    """The decay's bias is laid out heads x dim and its rate is one number per head: the oracle with the bias laid out
+    dim x heads, or with the rates of two heads exchanged, is far away."""
+    cfgd = config([cd(heads=3, kv_heads=3, dim=4, vdim=6)], bigram=None, side=0)
+
+    def spread(w):
+        for k in w:
+            if k.endswith("dt_bias"):
+                w[k] = torch.linspace(-4.0, 3.0, w[k].numel()).to(w[k].dtype)
+            if k.endswith("A_log"):
+                w[k] = torch.tensor([-3.0, 0.0, 1.5]).to(w[k].dtype)
+
+    t = toks(40, seed=14)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, tweak=spread)
+        want = m.expect(t)
+        turned = changed(m.weights, lambda k, v: v.view(3, 4).t().reshape(-1).contiguous() if k.endswith("dt_bias") else None)
+        assert gap(m.expect(t, weights=turned), want) > 1e-2
+        flipped = changed(m.weights, lambda k, v: v.flip(0) if k.endswith("A_log") else None)
+        assert gap(m.expect(t, weights=flipped), want) > 1e-2
+        m.check(m.run_cut("d", t, [17, 2, 1]), want, "decay layout")
+
+
+# ---------------------------------------------------------------------------------------------- far keys and edges
+@pytest.mark.parametrize("device", DEVICES)
+def test_far_key_among_hundreds(device):
+    """Attention without a window made sharp (query and key gains scaled up): single far keys carry the weight, and
+    their values arrive rotated by the distance.  Changing the second token moves logits 250 tokens later in the
+    oracle, and the engine agrees with it in prompts cut at page borders and in decoding."""
+    cfgd = config([att(heads=2, kv_heads=1, dim=8, vdim=6, window=None, dims=4, scale=0.5, cap=30.0)], bigram=None, side=0)
+    sharp = scaled([("q.norm", 2.5), ("k.norm", 2.5)])
+    t = toks(300, seed=10)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, max_tokens=320, tweak=sharp)
+        want = m.expect(t)
+        moved = list(t)
+        moved[1] = (moved[1] + 11) % VOCAB
+        assert gap_max(m.expect(moved), want, slice(250, None)) > 5e-2, "early tokens do not matter in this construction"
+        m.check(m.run_cut("a", t, [256, 1]), want, "prompt to a page border, then decoding")
+        m.check(m.run_cut("b", t, [32, 64, 33, 2, 97, 1]), want, "portions on and off page borders")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("window", [1, 2, 31, 32, 33, 40, 70])
+def test_window_edges(device, window):
+    """Sharp windowed attention: the key just inside the window counts and the one just outside does not, in prompts
+    and in decoding.  The oracle with a window one token larger or smaller is far from the design in the rows whose
+    strongest key sits at the edge (every row is judged against the design)."""
+    def cfg_w(w):
+        return config([att(heads=2, kv_heads=1, dim=8, vdim=6, window=w, scale=1.0, cap=50.0)], bigram=None, side=0)
+
+    sharp = scaled([("q.norm", 2.0), ("k.norm", 2.0)])
+    t = toks(110, seed=11)
+    for dtype in modes(device):
+        m = Model(cfg_w(window), device, dtype, tweak=sharp)
+        want = m.expect(t)
+        for other in (window + 1, window - 1):
+            if other >= 1:
+                assert gap_max(m.expect(t, cfg_w(other)), want, slice(window + 1, None)) > 1e-2, other
+        m.check(m.run_cut("p", t, [len(t)]), want, "prompt")
+        m.check(m.run_cut("d", t, [max(1, window - 1), 1]), want, "decoding over the edge")
+        m.check(m.run_cut("c", t, [window + 1, 2, 31, 1]), want, "portions over the edge")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_score_cap_and_value_rotation_matter(device):
+    """Large scores under a small cap, and a rotation base that turns values quickly: the oracle without the cap, with
+    another cap, or with values turned by another base is far away; the engine follows the design."""
+    def cfg_c(cap, base=20.0):
+        return config([att(heads=2, kv_heads=2, dim=6, vdim=8, window=20, dims=2, scale=1.5, cap=cap, base=base)],
+                      bigram=None, side=0)
+
+    t = toks(50, seed=15)
+    for dtype in modes(device):
+        m = Model(cfg_c(1.5), device, dtype, tweak=scaled([("q.norm", 2.0)]))
+        want = m.expect(t)
+        assert gap(m.expect(t, cfg_c(0)), want) > 1e-2 and gap(m.expect(t, cfg_c(3.0)), want) > 1e-2
+        assert gap(m.expect(t, cfg_c(1.5, base=2000.0)), want) > 1e-2
+        m.check(m.run_cut("c", t, [23, 2, 1]), want, "capped scores, rotated values")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_convolution_reaches_over_cuts(device):
+    """The short convolution with five taps: a portion's first rows read the tail that the step before left, also when
+    that step was shorter than the tail; the oracle with the current tap only is far away."""
+    cfgd = config([cd(conv=5, mlp=dense()), cd(heads=2, kv_heads=1, conv=5, mlp=moe())], bigram=None, side=0)
+    t = toks(40, seed=12)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype)
+        want = m.expect(t)
+        last_only = changed(m.weights, lambda k, v: torch.cat([v[:, :-1] * 0, v[:, -1:]], 1) if k.endswith(".conv") else None)
+        assert gap(m.expect(t, weights=last_only), want) > 5e-2
+        for cuts in ([2], [1], [3, 1, 1, 2, 6, 1], [4, 5, 1]):
+            m.check(m.run_cut("c", t, cuts), want, f"portions {cuts}")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_groups_limit_the_choice(device):
+    """A sharp router over four groups of which one is kept: the oracle without the limit is far away, the engine
+    follows the design."""
+    cfgd = config([att(mlp=moe(experts=8, top=2, groups=4, keep=1))], bigram=None, side=0)
+    t = toks(40, seed=13)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, tweak=scaled([("router", 4.0)]))
+        want = m.expect(t)
+        flat = copy.deepcopy(cfgd)
+        del flat["layers"][0]["mlp"]["router"]["groups"]
+        assert gap(m.expect(t, flat), want) > 1e-2
+        m.check(m.run_cut("r", t, [17, 2, 1]), want, "routing")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_token_inputs_take_their_layer_slice(device):
+    """Every layer reads its own columns of the side table, in every pass of a loop: the oracle with the slices of two
+    layers exchanged is far away."""
+    cfgd = config([att(mlp=dense()), cd()], bigram=None, side=5, loop=(1, 2, 2))
+    t = toks(30, seed=14)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, tweak=scaled([("side.embed", 3.0)]))
+        want = m.expect(t)
+        swapped = changed(m.weights, lambda k, v: torch.cat([v[:, 5:], v[:, :5]], 1) if k == "side.embed" else None)
+        assert gap(m.expect(t, weights=swapped), want) > 1e-2
+        m.check(m.run_cut("s", t, [11, 1]), want, "token inputs")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens(device):
+    """Positions 0, 1, 2: the pair table's last row, the convolution's empty history, a zero state and one-key
+    attention; as a one-token request, as single tokens from the start, and in a slot that held another sequence."""
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype, max_seqs=1)
+        m.run_cut("warm", toks(40, seed=15), [40])
+        for n in (1, 2, 3):
+            t = toks(n, seed=16 + n)
+            m.check(m.run_cut(f"n{n}", t, [1]), m.expect(t), f"{n} first tokens, one by one")
+            m.check(m.run_cut(f"w{n}", t, [n]), m.expect(t), f"{n} first tokens, at once")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding(device):
+    """Decoding runs over several pages and past the windows."""
+    t = toks(150, seed=20)
+    for dtype in modes(device):
+        m = Model(HYBRID, device, dtype)
+        m.check(m.run_cut("l", t, [5, 1]), m.expect(t), "long decoding")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,cfgd,rank", [
+    ("all ones", config([att(heads=1, kv_heads=1, dim=2, vdim=2, window=1, dims=2, mlp=dense(1)),
+                         cd(heads=1, kv_heads=1, dim=1, vdim=1, conv=1, mlp=moe(experts=1, top=1, ff=1, groups=1, keep=1))],
+                        width=2, vocab=7, bigram=(1, 1, 1), side=1, loop=(0, 2, 1)), (1, 1)),
+    ("odd sizes", config([cd(heads=6, kv_heads=2, dim=7, vdim=9, conv=4, mlp=moe(experts=9, top=4, ff=7, groups=3, keep=2)),
+                          att(heads=6, kv_heads=3, dim=14, vdim=10, window=13, dims=6, mlp=dense(17))], width=19, vocab=23,
+                         bigram=(13, 3, 5), side=3, loop=(0, 2, 2)), (7, 11)),
+    ("sizes that vector loads and the MFMA attention like", config(
+        [att(heads=8, kv_heads=2, dim=64, vdim=32, window=48, dims=32, mlp=moe(experts=8, top=2, ff=64, groups=2, keep=1)),
+         cd(heads=4, kv_heads=2, dim=32, vdim=16, conv=4, mlp=dense(128)),
+         att(heads=2, kv_heads=1, dim=32, vdim=64, window=None, dims=32, cap=0)], width=64, vocab=96, bigram=(64, 17, 3),
+        side=8), (8, 16)),
+    ("wide heads", config([att(heads=2, kv_heads=1, dim=136, vdim=72, window=20, dims=100),
+                           cd(heads=2, kv_heads=1, dim=136, vdim=72)], width=48, vocab=50), (3, 9)),
+    ("projections on the tiled-layout GEMMs", config(
+        [att(heads=8, kv_heads=4, dim=128, vdim=128, window=40, dims=64, mlp=dense(2048)),
+         cd(heads=8, kv_heads=4, dim=128, vdim=128, mlp=moe(experts=4, top=2, ff=256, groups=2, keep=2))],
+        width=1024, vocab=1024, bigram=(4093, 1024, 1), side=16, loop=(1, 2, 2)), (24, 40)),
+])
+def test_other_sizes(device, name, cfgd, rank):
+    vocab = cfgd["vocab"]
+    t = toks(41, vocab=vocab, seed=21)
+    for dtype in modes(device):
+        m = Model(cfgd, device, dtype, rank=rank)
+        m.check(m.run_cut("x", t, [len(t)]), m.expect(t), name + ", whole")
+        m.check(m.run_cut("y", t, [7, 2, 1]), m.expect(t), name + ", portions and decoding")
+
+
+@pytest.mark.gpu
+def test_long_prompt_of_many_tiles():
+    """Six hundred tokens on the GPU: prompt-sized expert tiles, attention tiles over many pages, windows inside, long
+    walks of the delta rule."""
+    cfgd = config([att(heads=4, kv_heads=2, dim=32, vdim=32, window=100, dims=16, mlp=moe(experts=8, top=2, ff=64, groups=4, keep=2)),
+                   cd(heads=4, kv_heads=2, dim=32, vdim=32, conv=4, mlp=dense(128))], width=64, vocab=200, side=8,
+                  loop=(0, 2, 2))
+    t = toks(600, vocab=200, seed=22)
+    for dtype in (torch.float32, torch.bfloat16):
+        m = Model(cfgd, "cuda", dtype, max_tokens=640)
+        want = m.expect(t)
+        m.check(m.run_cut("a", t, [560, 1]), want, "prompt, then decoding")
+        m.check(m.run_cut("b", t, [300, 3, 257, 1]), want, "portions")
+
+
+# ---------------------------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_the_scheduler(device):
+    """add_request + step: admission, chunked prompt passes (a 16-token budget), mixed steps, decode with sampling at
+    temperature 0 (the sampled token becomes the next one's predecessor on the device), slot release.  Each generated
+    token is the oracle's argmax given the tokens before it (a step whose two best logits are closer than the
+    tolerance is not judged)."""
+    m = Model(HYBRID, device, torch.float32, max_tokens=512, max_seqs=3)
+    eng = LLMEngine(m.runner, eos_id=-1, prefill_budget=16, idle_prefill_budget=16)
+    prompts = {"g0": toks(19, seed=23), "g1": toks(40, seed=24), "g2": toks(3, seed=25), "g3": toks(33, seed=26)}
+    for cid, p in prompts.items():
+        eng.add_request(cid, p, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    out = {cid: [] for cid in prompts}
+    for ev in eng.run_until_idle():
+        if not ev.done:
+            out[ev.conversation_id].append(ev.token_id)
+    for cid, p in prompts.items():
+        assert len(out[cid]) == 12, (cid, out[cid])
+        logits = m.expect(p + out[cid])
+        for i, tok in enumerate(out[cid]):
+            row = logits[len(p) + i - 1]
+            top = torch.topk(row, 2).values
+            if float(top[0] - top[1]) > 1e-3 * float(row.abs().max()):
+                assert tok == int(row.argmax()), f"{cid}: token {i} is {tok}, the oracle says {int(row.argmax())}"
+    assert eng.alloc.num_free == eng.alloc.num_blocks
+
+
+@pytest.mark.gpu
+def test_decode_graphs_match_eager():
+    """The captured decode step replayed over several steps (with eager work between the replays) gives the eager
+    step's logits; the previous token is carried inside the graph."""
+    m = Model(HYBRID, "cuda", torch.bfloat16)
+    t = toks(60, seed=27)
+    eager = m.run_cut("e", t, [20, 1])
+    m.runner.use_graphs = True
+    m.runner.capture()
+    assert m.runner.graphs
+    graphed = m.run_cut("g", t, [20, 1])
+    assert torch.allclose(eager, graphed, atol=1e-5, rtol=1e-5)
+    m.check(graphed, m.expect(t), "graph replays")
+
+
+def test_config_round_trip_and_registry(tmp_path):
+    cfg = MurulornConfig.from_dict(HYBRID)
+    again = MurulornConfig.from_dict(cfg.to_dict())
+    assert again.layers == cfg.layers and again == cfg
+    assert [r.layer for r in cfg.runs()] == [0, 1, 2, 1, 2, 3]
+    assert [r.pass_no for r in cfg.runs()] == [-1, 0, -1, 1, -1, -1]
+    bare = MurulornConfig.from_dict(config([att()], **BARE))
+    assert bare.bigram is None and bare.side_dim == 0 and bare.loop_times == 0
+    assert MurulornConfig.from_dict(bare.to_dict()) == bare and set(tensor_shapes(bare)) == {
+        "embed", "final.norm", "l0.norm1", "l0.norm1b", "l0.mix.q", "l0.mix.k", "l0.mix.v", "l0.mix.q.norm", "l0.mix.k.norm",
+        "l0.mix.g", "l0.mix.o"}
+    from safetensors.torch import save_file
+
+    (tmp_path / "config.json").write_text(json.dumps(HYBRID))
+    weights = init_weights(cfg, seed=3, rank=(5, 3))
+    save_file({k: v.contiguous() for k, v in weights.items()}, str(tmp_path / "model.safetensors"))
+    fam, cfg2, path = registry.resolve(str(tmp_path))
+    assert fam.name == "murulorn" and cfg2.layers == cfg.layers and cfg2.width == cfg.width and path == str(tmp_path)
+    w = registry.load_weights(fam, cfg2, path, device="cpu", dtype=torch.float32)
+    assert w.layers[1].mlp.up.shape == (6, 9, 26) and w.layers[1].mix.a2.shape == (4 * 6, 5) and w.layers[1].mix.g2.shape == (40, 3)
+    assert w.head is w.embed and w.bigram.shape == (38, 26) and w.loop_in.shape == (26, 52) and w.layers[2].side.col0 == 14
+    assert torch.allclose(w.layers[0].norm1, 1.0 + weights["l0.norm1"].float())
+    assert set(tensor_shapes(cfg)) == set(weights)
+    assert registry.resolve("murulorn-tiny")[0].name == "murulorn"
+    assert cfg.cache_bytes_per_token() > 0 and cfg.state_bytes_per_sequence() > 0
+    bad = dict(weights)
+    bad["l0.mix.q"] = bad["l0.mix.q"][:-1]
+    with pytest.raises(ValueError):
+        convert_murulorn(cfg, bad)
+    with pytest.raises(ValueError):
+        MurulornConfig.from_dict(config([att(mlp=moe(experts=6, top=5, groups=3, keep=2))]))
+    with pytest.raises(ValueError):
+        MurulornConfig.from_dict(config([att(vdim=7)]))
+
+
+def test_portion_without_a_predecessor_is_refused():
+    """A portion that starts inside a sequence needs the token before it: from the caller, or from the slot's latest
+    portion; otherwise the runner refuses instead of hashing a wrong pair."""
+    m = Model(HYBRID, "cpu")
+    t = toks(12, seed=28)
+    with pytest.raises(ValueError):
+        m.runner.prefill([PrefillSeq(slot=1, tokens=t[6:], start_pos=6, block_table=[1], last_chunk=False)], 0)
+    m.runner.prefill([PrefillSeq(slot=0, tokens=t[:6], start_pos=0, block_table=[0], last_chunk=False)], 0)
+    m.runner.prefill([PrefillSeq(slot=0, tokens=t[6:], start_pos=6, block_table=[0], last_chunk=False, want=(5,))], 0)
+    m.check(m.runner.kept_logits, m.expect(t)[-1:], "the slot's remembered token")
+
+
+def test_serving_builds_the_family_by_name():
+    """The serving launcher's engine builder resolves the family through the registry and generates with it."""
+    from distributed_sse_for_llm_response_amd.serving.app import build_engine
+    from distributed_sse_for_llm_response_amd.serving.config import ServeConfig
+
+    eng, _ = build_engine(ServeConfig(model="murulorn-tiny", engine="cpu"))
+    eng.add_request("c1", [5, 6, 7, 8, 9, 10], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    eng.add_request("c2", [11, 12], SamplingParams(temperature=0.8, max_tokens=3, ignore_eos=True))
+    ev = eng.run_until_idle()
+    assert sum(1 for e in ev if e.conversation_id == "c1" and not e.done) == 4
+    assert sum(1 for e in ev if e.conversation_id == "c2" and not e.done) == 3

@@ -68,7 +68,7 @@ def main():
                          "STUB_STEP_MS instead of the model (router/bus/SSE/client at N GPUs' token rate)")
     ap.add_argument("--families", default="",
                     help="comma-separated model names: instead of the headline workload, print prompt and decode "
-                         "throughput of each on its runner (e.g. muderax-mid,mistral-mid); one GPU, --streams, "
+                         "throughput of each on its runner (e.g. murulorn-mid,surodra-mid,mistral-mid); one GPU, --streams, "
                          "--prompt-len, --steps, --warmup apply")
     args = ap.parse_args()
     if args.families:

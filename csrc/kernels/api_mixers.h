@@ -160,9 +160,31 @@ struct AddNormParams {
   float eps;
 };
 
+// A per-layer token input in one launch (decode-sized steps): stream += norm(y) * g_add; g = gelu_tanh(gate_w x) *
+// table[id, col0 : col0 + F] on the rounded stream x; stream += norm(proj_w g) * side_norm; out = norm(stream) * g_out.
+struct TokenSideParams {
+  const float* y;        // [M * nsum, W] pending sublayer output or null
+  int nsum;
+  const float* g_add;    // [W]
+  float* resid;          // [M, W] fp32
+  const int* ids;        // [M]
+  const void* table;     // [vocab, ldt] element type
+  int vocab, ldt, col0;
+  const void* gate_w;    // [F, W] element type
+  const void* proj_w;    // [W, F] element type
+  const float* side_norm;  // [W]
+  const float* g_out;    // [W] or null: out = the stream itself
+  void* out;             // rows ldo apart, element type, or null
+  float* out32;          // [M, W] or null
+  int ldo;
+  int M, W, F, f32;
+  float eps;
+};
+
 }  // namespace dsse
 
 extern "C" {
+hipError_t dsse_token_side_rows(const dsse::TokenSideParams* p, hipStream_t st);
 hipError_t dsse_embed_pair_rows(const dsse::EmbedPairParams* p, hipStream_t st);
 hipError_t dsse_add_norm_rows(const dsse::AddNormParams* p, hipStream_t st);
 // out [M, F] = gelu_tanh(x) * table[ids, col0 : col0 + F] (table rows ldt apart)

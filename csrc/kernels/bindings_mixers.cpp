@@ -637,7 +637,60 @@ void token_gate_rows(const Tensor& x, const Tensor& ids, const Tensor& table, in
                                       elem(table, "table"), cur_stream()));
 }
 
+void token_side_rows(const OptTensor& y, int64_t nsum, const OptTensor& g_add, Tensor& resid, const Tensor& ids,
+                     const Tensor& table, int64_t col0, const Tensor& gate_w, const Tensor& proj_w, const Tensor& side_norm,
+                     const OptTensor& g_out, double eps, const OptTensor& out, const OptTensor& out32) {
+  f32t(resid, "resid");
+  i32(ids, "ids");
+  gpu(table, "table");
+  gpu(gate_w, "gate_w");
+  gpu(proj_w, "proj_w");
+  TORCH_CHECK(resid.dim() == 2 && nsum >= 1 && gate_w.dim() == 2 && proj_w.dim() == 2 && table.dim() == 2, "shapes");
+  dsse::TokenSideParams p{};
+  p.M = (int)resid.size(0), p.W = (int)resid.size(1), p.F = (int)gate_w.size(0);
+  TORCH_CHECK(gate_w.size(1) == p.W && proj_w.size(0) == p.W && proj_w.size(1) == p.F, "gate_w [F, W], proj_w [W, F]");
+  TORCH_CHECK(gate_w.scalar_type() == proj_w.scalar_type() && table.scalar_type() == gate_w.scalar_type(),
+              "gate_w, proj_w and table share the element type");
+  TORCH_CHECK(col0 >= 0 && col0 + p.F <= table.size(1) && ids.numel() >= p.M, "table must hold col0 + F columns, one id per row");
+  TORCH_CHECK((int64_t)(p.W + p.F + 8) * 4 <= 64 * 1024, "row too wide for the one-launch form");
+  p.f32 = elem(gate_w, "gate_w");
+  p.resid = resid.data_ptr<float>();
+  p.nsum = (int)nsum;
+  if (y.has_value()) {
+    f32t(*y, "y");
+    TORCH_CHECK(y->numel() == (int64_t)p.M * nsum * p.W && g_add.has_value(), "y must hold M * nsum rows of W, with its gain");
+    p.y = y->data_ptr<float>();
+    p.g_add = opt_f32(g_add, "g_add", p.W);
+  }
+  p.ids = ids.data_ptr<int>();
+  p.table = table.data_ptr();
+  p.vocab = (int)table.size(0), p.ldt = (int)table.size(1), p.col0 = (int)col0;
+  p.gate_w = gate_w.data_ptr();
+  p.proj_w = proj_w.data_ptr();
+  f32t(side_norm, "side_norm");
+  TORCH_CHECK(side_norm.numel() == p.W, "side_norm must be [W]");
+  p.side_norm = side_norm.data_ptr<float>();
+  p.g_out = opt_f32(g_out, "g_out", p.W);
+  if (out.has_value()) {
+    gpu(*out, "out", false);
+    TORCH_CHECK(out->scalar_type() == gate_w.scalar_type() && out->dim() == 2 && out->size(0) == p.M && out->size(1) == p.W &&
+                    (p.W == 1 || out->stride(1) == 1) && out->stride(0) >= p.W,
+                "out must be [M, W] in the weights' type with unit column stride");
+    p.out = out->data_ptr();
+    p.ldo = (int)out->stride(0);
+  }
+  if (out32.has_value()) {
+    f32t(*out32, "out32");
+    TORCH_CHECK(out32->numel() == (int64_t)p.M * p.W, "out32 must be [M, W]");
+    p.out32 = out32->data_ptr<float>();
+  }
+  p.eps = (float)eps;
+  DSSE_CHECK_HIP(dsse_token_side_rows(&p, cur_stream()));
+}
+
 TORCH_LIBRARY_FRAGMENT(dsse, m) {
+  m.def("token_side_rows(Tensor? y, int nsum, Tensor? g_add, Tensor(a!) resid, Tensor ids, Tensor table, int col0, "
+        "Tensor gate_w, Tensor proj_w, Tensor side_norm, Tensor? g_out, float eps, Tensor(b!)? out, Tensor(c!)? out32) -> ()");
   m.def("stream_mix(Tensor? y, int nsum, float mult, Tensor(a!) streams, Tensor? ids, Tensor? embed, float embed_scale, "
         "Tensor? out_w, Tensor? mix, Tensor? in_w, Tensor? norm_w, float eps, Tensor(b!)? h, Tensor(c!)? total) -> ()");
   m.def("act_rows(Tensor x, Tensor(a!) out, int kind, Tensor? params=None, Tensor? gate=None) -> ()");
@@ -674,6 +727,7 @@ TORCH_LIBRARY_IMPL(dsse, CUDA, m) {
   m.impl("embed_pair_rows", &embed_pair_rows);
   m.impl("add_norm_rows", &add_norm_rows);
   m.impl("token_gate_rows", &token_gate_rows);
+  m.impl("token_side_rows", &token_side_rows);
   m.impl("stream_step", &stream_step);
   m.impl("gated_act", &gated_act);
   m.impl("norm_rope_rows", &norm_rope_rows);

@@ -8,6 +8,9 @@
 //                    out = resid / rms(resid) * g_out (or resid itself): the add of one sublayer and the norm of the next
 //                    in one pass over the row, the row held in registers between its two statistics
 //   token_gate_rows  out = gelu_tanh(x) * table[id, col0 : col0 + F]
+//   token_side_rows  a whole per-layer token input for decode-sized steps in ONE launch: the pending add + norm, the
+//                    gate's few dot products per row, the table slice, the back-projection, its norm and add, and the
+//                    next sublayer's norm -- five launches of latency-sized kernels otherwise
 //
 // Everything is computed in fp32; only outputs of the element type are rounded.
 #include "api_mixers.h"
@@ -178,6 +181,116 @@ __global__ __launch_bounds__(256) void token_gate_rows_kernel(const float* x, in
   }
 }
 
+// One workgroup per row.  The row lives in LDS: first the rounded stream (what the gate's projection reads), then the
+// back-projection's output.  A wave owns every fourth gate column (lanes stride over the width, 16-byte loads); a
+// thread owns every 256th channel of the back-projection (its weight row is F contiguous numbers).
+template <typename T>
+__global__ __launch_bounds__(256) void token_side_rows_kernel(TokenSideParams p) {
+  extern __shared__ float side_sm[];
+  float* xs = side_sm;      // [W]
+  float* gs = xs + p.W;     // [F]
+  float* red = gs + p.F;    // [4]
+  constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
+  const int64_t row = blockIdx.x;
+  const int W = p.W, F = p.F;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* resid = p.resid + row * W;
+  if (p.y) {
+    const float* y = p.y + row * p.nsum * W;
+    float sy = 0.f;
+    for (int d = threadIdx.x; d < W; d += 256) {
+      float v = 0.f;
+      for (int s = 0; s < p.nsum; ++s) v += y[(int64_t)s * W + d];
+      xs[d] = v;
+      sy += v * v;
+    }
+    sy = block_sum256(sy, red);
+    const float inv = 1.0f / sqrtf(sy / (float)W + p.eps);
+    for (int d = threadIdx.x; d < W; d += 256) {
+      const float r = resid[d] + xs[d] * inv * p.g_add[d];
+      resid[d] = r;
+      xs[d] = (float)(T)r;
+    }
+  } else {
+    for (int d = threadIdx.x; d < W; d += 256) xs[d] = (float)(T)resid[d];
+  }
+  __syncthreads();
+  int id = p.ids[row];
+  id = (unsigned)id < (unsigned)p.vocab ? id : 0;
+  const T* trow = reinterpret_cast<const T*>(p.table) + (int64_t)id * p.ldt + p.col0;
+  const T* gate_w = reinterpret_cast<const T*>(p.gate_w);
+  const bool vw = W % VEC == 0;
+  for (int j = wave; j < F; j += 4) {
+    const T* gw = gate_w + (int64_t)j * W;
+    float s = 0.f;
+    if (vw) {
+      for (int d = lane * VEC; d < W; d += 64 * VEC) {
+        if constexpr (VEC == 8) {
+          const bf16x8 t = *reinterpret_cast<const bf16x8*>(gw + d);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) s += (float)t[e] * xs[d + e];
+        } else {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(gw + d);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s += t[e] * xs[d + e];
+        }
+      }
+    } else {
+      for (int d = lane; d < W; d += 64) s += (float)gw[d] * xs[d];
+    }
+    s = wave_sum(s);
+    if (lane == 0) gs[j] = (float)(T)(gelu_tanh_f(s) * (float)trow[j]);
+  }
+  __syncthreads();  // the gate columns are complete, and nobody reads the rounded stream any more
+  const T* proj_w = reinterpret_cast<const T*>(p.proj_w);
+  const bool vf = F % VEC == 0;
+  float sy = 0.f;
+  for (int d = threadIdx.x; d < W; d += 256) {
+    const T* pw = proj_w + (int64_t)d * F;
+    float v = 0.f;
+    if (vf) {
+      for (int j = 0; j < F; j += VEC) {
+        if constexpr (VEC == 8) {
+          const bf16x8 t = *reinterpret_cast<const bf16x8*>(pw + j);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v += (float)t[e] * gs[j + e];
+        } else {
+          const f32x4 t = *reinterpret_cast<const f32x4*>(pw + j);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v += t[e] * gs[j + e];
+        }
+      }
+    } else {
+      for (int j = 0; j < F; ++j) v += (float)pw[j] * gs[j];
+    }
+    xs[d] = v;  // this thread's own channel: read back below by the same thread
+    sy += v * v;
+  }
+  sy = block_sum256(sy, red);
+  const float inv = 1.0f / sqrtf(sy / (float)W + p.eps);
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < W; d += 256) {
+    const float r = resid[d] + xs[d] * inv * p.side_norm[d];
+    resid[d] = r;
+    xs[d] = r;
+    ss += r * r;
+  }
+  if (!p.out && !p.out32) return;  // uniform
+  float inv2 = 1.0f;
+  if (p.g_out) {
+    ss = block_sum256(ss, red);
+    inv2 = 1.0f / sqrtf(ss / (float)W + p.eps);
+  }
+  T* out = p.out ? reinterpret_cast<T*>(p.out) + row * p.ldo : nullptr;
+  float* out32 = p.out32 ? p.out32 + row * W : nullptr;
+  for (int d = threadIdx.x; d < W; d += 256) {
+    float r = xs[d];
+    if (p.g_out) r = r * inv2 * p.g_out[d];
+    if (out) out[d] = (T)r;
+    if (out32) out32[d] = r;
+  }
+}
+
 template <typename OutT>
 void launch_add_norm(const AddNormParams& p, hipStream_t st) {
   const dim3 g(p.M), b(256);
@@ -219,5 +332,14 @@ extern "C" hipError_t dsse_token_gate_rows(const float* x, int ldx, const int* i
   else
     hipLaunchKernelGGL(dsse::token_gate_rows_kernel<bf16>, dim3(blocks), dim3(256), 0, st, x, ldx, ids,
                        reinterpret_cast<const bf16*>(table), vocab, ldt, col0, reinterpret_cast<bf16*>(out), M, F);
+  return hipGetLastError();
+}
+
+extern "C" hipError_t dsse_token_side_rows(const dsse::TokenSideParams* p, hipStream_t st) {
+  if (p->M <= 0) return hipSuccess;
+  const size_t lds = (size_t)(p->W + p->F + 8) * sizeof(float);
+  if (p->nsum < 1 || (p->y && !p->g_add) || p->F < 1 || lds > 64 * 1024) return hipErrorInvalidValue;
+  if (p->f32) hipLaunchKernelGGL(dsse::token_side_rows_kernel<float>, dim3(p->M), dim3(256), lds, st, *p);
+  else hipLaunchKernelGGL(dsse::token_side_rows_kernel<bf16>, dim3(p->M), dim3(256), lds, st, *p);
   return hipGetLastError();
 }

@@ -81,22 +81,24 @@ __global__ __launch_bounds__(256) void gemm_rm_kernel(GemmRmParams p) {
     }
 }
 
-// Up to 16 rows (decode buckets, per-head and per-block slices): a workgroup owns one 16 x 16 output tile and its four
-// waves split the K axis (k-steps w, w + 4, ...), meeting in LDS.  Four times the workgroups of a 16 x 64 tile and a
-// quarter of the dependent k-steps per wave: these launches are latency-bound, not bandwidth-bound.
+// Up to 16 rows (decode buckets, per-head and per-block slices), or many rows of a NARROW output (a router's logits, a
+// few-column gate: up to 64 columns): a workgroup owns one 16 x 16 output tile and its four waves split the K axis
+// (k-steps w, w + 4, ...), meeting in LDS.  Four times the workgroups of a 16 x 64 tile and a quarter of the dependent
+// k-steps per wave: these launches are latency-bound, not bandwidth-bound -- a narrow output leaves the 64 x 64 tiles
+// of the general kernel a handful of workgroups that each walk the whole K axis.
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_rm_skinny_kernel(GemmRmParams p) {
   using F = Frag<T>;
   __shared__ float red[4 * 4 * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int col0 = blockIdx.x * 16;
+  const int col0 = blockIdx.x * 16, row0 = blockIdx.y * 16;
   const int z = blockIdx.z;
   const T* X = reinterpret_cast<const T*>(p.x) + (int64_t)z * p.xbs;
   const T* W = reinterpret_cast<const T*>(p.w) + (int64_t)z * p.wbs;
   const T* bias = p.bias ? reinterpret_cast<const T*>(p.bias) + (int64_t)z * p.bbs : nullptr;
-  const bool xv = r < p.M, wv = col0 + r < p.N;
-  const T* xr = X + (int64_t)(xv ? r : 0) * p.ldx;
+  const bool xv = row0 + r < p.M, wv = col0 + r < p.N;
+  const T* xr = X + (int64_t)(xv ? row0 + r : 0) * p.ldx;
   const T* wr = W + (int64_t)(wv ? col0 + r : 0) * p.ldw;
   const bool vx = p.vecx != 0, vw = p.vecw != 0;
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(256) void gemm_rm_skinny_kernel(GemmRmParams p) {
   const float bv = bias ? (float)bias[col] : 0.0f;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const int row = 4 * g + e;
+    const int row = row0 + 4 * g + e;
     if (row >= p.M) continue;
     float v = red[e * 64 + lane] + red[(4 + e) * 64 + lane] + red[(8 + e) * 64 + lane] + red[(12 + e) * 64 + lane] + bv;
     if (p.act == 1) v = gelu_tanh(v);
@@ -132,8 +134,8 @@ hipError_t launch(const GemmRmParams& p, hipStream_t st) {
 
 template <typename T>
 hipError_t dispatch(const GemmRmParams& p, hipStream_t st) {
-  if (p.M <= 16) {
-    hipLaunchKernelGGL(gemm_rm_skinny_kernel<T>, dim3((p.N + 15) / 16, 1, p.batch), dim3(256), 0, st, p);
+  if (p.M <= 16 || (p.N <= 64 && p.K >= 256)) {
+    hipLaunchKernelGGL(gemm_rm_skinny_kernel<T>, dim3((p.N + 15) / 16, (p.M + 15) / 16, p.batch), dim3(256), 0, st, p);
     return hipGetLastError();
   }
   if (p.M >= 256 && p.N >= 256) return launch<T, 4, 4, 2, 2>(p, st);

@@ -739,7 +739,7 @@ class LayeredRunner(RunnerBase):
 
     def _bracket_buffers(self, M: int) -> dict:
         """Scratch of a step of M rows, each sized for the widest layer: `big` the fused projection's fp32 output, `cv`
-        the convolution's, `z` the per-channel decays, `gz` the output gate's pre-activations, `qa` the attention's
+        the convolution's, `z` the per-channel decays beside the output gate's pre-activations, `qa` the attention's
         normed and rotated queries, `o` the recurrence's heads, `ao` a mixer's gated output in the element type, `up` /
         `h` the dense feed-forward's hidden row, `hn` the fp32 normed row a router reads, `cat` [stream | embedding
         output] for the projection that opens a loop pass, `sg` / `sh` the token input's gate, and the experts' lists."""
@@ -749,7 +749,7 @@ class LayeredRunner(RunnerBase):
         f32 = dict(device=dev, dtype=torch.float32)
         el = dict(device=dev, dtype=self.dtype)
         W = cfg.width
-        big = cv = z = gz = qa = o = ff = 1
+        big = cv = z = qa = o = ff = 1
         moe = []
         for i, L in enumerate(cfg.layers):
             m = L.mixer
@@ -758,14 +758,13 @@ class LayeredRunner(RunnerBase):
             if L.kind == "attention":
                 qa = max(qa, m.heads * m.dim)
             else:
-                cv, z = max(cv, 2 * m.kv_heads * m.dim + m.heads * m.vdim), max(z, m.heads * m.dim)
-                gz = max(gz, m.heads * m.vdim)
+                cv, z = max(cv, 2 * m.kv_heads * m.dim + m.heads * m.vdim), max(z, m.heads * (m.dim + m.vdim))
             if isinstance(L.mlp, SoftmaxRoutedSpec):
                 moe.append(L.mlp)
             elif L.mlp is not None:
                 ff = max(ff, L.mlp.ff)
         d = {"big": torch.zeros(M * big, **f32), "cv": torch.zeros(M * cv, **f32), "z": torch.zeros(M * z, **f32),
-             "gz": torch.zeros(M * gz, **f32), "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32),
+             "qa": torch.zeros(M * qa, **f32), "o": torch.zeros(M * o, **f32),
              "ao": torch.zeros(M * o, **el), "up": torch.zeros(M * ff, **f32), "h": torch.zeros(M * ff, **el),
              "hn": torch.zeros(M, W, **f32) if moe else None,
              "cat": torch.zeros(M, 2 * W, **el) if cfg.loop_times > 0 else None,
@@ -786,7 +785,8 @@ class LayeredRunner(RunnerBase):
         """Every layer run over M packed rows.  Between sublayers ONE add_norm_rows adds the finished sublayer's normed
         output to the stream and norms the stream for the next one (or rounds it, for the token input's gate and for
         the projection that opens a loop pass); the last output is added before the head's norm.  `pending` is the
-        sublayer output that is not in the stream yet: (rows, parts per row, gain of its norm)."""
+        sublayer output that is not in the stream yet: (rows, parts per row, gain of its norm).  Decode-sized steps
+        run a layer's token input as ONE launch (token_side_rows) that also writes the next sublayer's input."""
         from ..models.murulorn import SoftmaxRoutedSpec
 
         cfg, w, eps = self.cfg, self.w, self.cfg.eps
@@ -799,13 +799,18 @@ class LayeredRunner(RunnerBase):
         ops.embed_pair_rows(ids, prev_rows, pos, w.embed, w.bigram, bg.mul_prev if bg else 0, bg.mul_cur if bg else 0,
                             bg.buckets if bg else 1, d["resid"], cat[:, W:] if cat is not None else None, prev_out, keep)
         pending = (None, 1, None)
-        for run in self.runs:
+        ready = False  # the next sublayer's input (xb, or the stream's half of cat) is already written
+        fused_side = cfg.side_dim > 0 and ops.token_side_fits(M, W, cfg.side_dim)
+        for n, run in enumerate(self.runs):
             L, Lw = cfg.layers[run.layer], w.layers[run.layer]
             if run.pass_no >= 0:  # a pass of the looped span opens: stream <- W_in [stream | embedding output]
-                ops.add_norm_rows(*pending, d["resid"], None, eps, cat[:, :W])
+                if not ready:
+                    ops.add_norm_rows(*pending, d["resid"], None, eps, cat[:, :W])
                 self._lin(cat, w.loop_in, w.loop_in_t, d["resid"])
-                pending = (None, 1, None)
-            ops.add_norm_rows(*pending, d["resid"], Lw.norm1, eps, d["xb"])
+                pending, ready = (None, 1, None), False
+            if not ready:
+                ops.add_norm_rows(*pending, d["resid"], Lw.norm1, eps, d["xb"])
+            ready = False
             getattr(self, "_" + L.kind + "_bracket")(run.index, L.mixer, Lw.mix, M, d, pos, slots, groups)
             pending = (d["y"], 1, Lw.norm1b)
             if L.mlp is not None:
@@ -818,15 +823,25 @@ class LayeredRunner(RunnerBase):
                     pending = (d["y"], 1, Lw.norm2b)
             if Lw.side is not None:  # the layer's token input reads the stream after the feed-forward
                 sd = Lw.side
-                F = sd.gate.shape[0]
-                sg, sh = d["sg"][:M * F].view(M, F), d["sh"][:M * F].view(M, F)
-                ops.add_norm_rows(*pending, d["resid"], None, eps, d["xb"])
-                ops.gemm_rm(d["xb"], sd.gate, sg)
-                ops.token_gate_rows(sg, ids, w.side_embed, sd.col0, sh)
-                ops.gemm_rm(sh, sd.proj, d["y"])
-                pending = (d["y"], 1, sd.norm)
+                if fused_side:  # decode-sized steps: one launch, which also makes the next sublayer's input
+                    nxt = self.runs[n + 1] if n + 1 < len(self.runs) else None
+                    g_out, out = None, None
+                    if trace is None and nxt is not None:
+                        g_out, out = (None, cat[:, :W]) if nxt.pass_no >= 0 else (w.layers[nxt.layer].norm1, d["xb"])
+                    ops.token_side_rows(*pending, d["resid"], ids, w.side_embed, sd.col0, sd.gate, sd.proj, sd.norm, g_out,
+                                        eps, out)
+                    pending, ready = (None, 1, None), out is not None
+                else:
+                    F = sd.gate.shape[0]
+                    sg, sh = d["sg"][:M * F].view(M, F), d["sh"][:M * F].view(M, F)
+                    ops.add_norm_rows(*pending, d["resid"], None, eps, d["xb"])
+                    ops.gemm_rm(d["xb"], sd.gate, sg)
+                    ops.token_gate_rows(sg, ids, w.side_embed, sd.col0, sh)
+                    ops.gemm_rm(sh, sd.proj, d["y"])
+                    pending = (d["y"], 1, sd.norm)
             if trace is not None:
-                ops.add_norm_rows(*pending, d["resid"], None, eps)
+                if pending[0] is not None:
+                    ops.add_norm_rows(*pending, d["resid"], None, eps)
                 pending = (None, 1, None)
                 trace.append(d["resid"].clone())
         if pending[0] is not None:
@@ -865,31 +880,29 @@ class LayeredRunner(RunnerBase):
     def _channel_delta_bracket(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
         """Gated delta rule with a decay per head and key channel: ONE fused GEMM [q | k | v | b | a1 | g1] (fp32 out)
         -> conv_state over q | k | v (SiLU; slot tail) -> unit q, k per head -> the decay's and the gate's second
-        projections in fp32 -> gate_math (one rate per head, one bias per head and channel) -> matrix_scan (delta rule
+        projections in fp32 as one block-diagonal product -> gate_math (one rate per head, one bias per head and channel) -> matrix_scan (delta rule
         with per-channel decay; slot state) -> per-head RMS norm times the sigmoid gate -> output GEMM."""
         H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
         C = 2 * G * D + H * V
-        ra, rg = Lw.a2.shape[1], Lw.g2.shape[1]
         big = d["big"][:M * Lw.n_big].view(M, Lw.n_big)
         cv = d["cv"][:M * C].view(M, C)
         self._lin(d["xb"], Lw.big, Lw.big_t, big)
         for g in groups:
             ops.conv_state(big[:, :C], Lw.conv, None, self.state.tail.get(ri), g["qs"], g["ql"], g["ctx"], g["ss"], cv,
-                           None, None, 1)
+                           None, None, 1, g["qt"] == 1)
         q, k, v = self._cols(cv, 0, G, D), self._cols(cv, G * D, G, D), self._cols(cv, 2 * G * D, H, V)
         ops.norm_rope_rows(q, None, pos, None, q, None, 2, UNIT_EPS, D ** -0.5)
         ops.norm_rope_rows(k, None, pos, None, k, None, 2, UNIT_EPS, 1.0)
         beta = big[:, C:C + H]
         ops.gate_math(beta, 1)
-        z = d["z"][:M * H * D].view(M, H * D)
-        gz = d["gz"][:M * H * V].view(M, H * V)
-        ops.gemm_rm(big[:, C + H:C + H + ra], Lw.a2, z)
+        zz = d["z"][:M * H * (D + V)].view(M, H * (D + V))
+        z, gz = zz[:, :H * D], zz[:, H * D:]
+        ops.gemm_rm(big[:, C + H:C + H + Lw.ra + Lw.rg], Lw.ag2, zz)
         ops.gate_math(z, 0, Lw.a_log, Lw.dt_bias)
-        ops.gemm_rm(big[:, C + H + ra:C + H + ra + rg], Lw.g2, gz)
         o = d["o"][:M * H * V].view(M, H, V)
         for g in groups:
-            ops.matrix_scan(q, k, v, z.view(M, H, D), beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"], g["ss"], o,
-                            1.0)
+            ops.matrix_scan(q, k, v, z.unflatten(1, (H, D)), beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"],
+                            g["ss"], o, 1.0)
         ao = d["ao"][:M * H * V].view(M, H * V)
         ops.gated_head_norm(o, Lw.norm, gz, self.cfg.eps, ao, 1)
         self._lin(ao, Lw.o, Lw.o_t, d["y"])

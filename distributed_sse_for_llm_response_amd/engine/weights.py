@@ -711,8 +711,10 @@ class ChannelDeltaWeights:
     conv: torch.Tensor       # [2 G D + H V, taps] fp32: the taps of q | k | v
     a_log: torch.Tensor      # [H] fp32
     dt_bias: torch.Tensor    # [H D] fp32
-    a2: torch.Tensor         # [H D, ra] fp32 (its input is the fp32 output of a1)
-    g2: torch.Tensor         # [H V, rg] fp32
+    ag2: torch.Tensor        # [H D + H V, ra + rg] fp32, block-diagonal: the decay's and the gate's second projections
+                             # as ONE product on the adjacent fp32 outputs of a1 and g1 (rows [a2 | 0] then [0 | g2])
+    ra: int                  # inner widths of the two pairs
+    rg: int
     norm: torch.Tensor       # [V] fp32
     o: torch.Tensor          # [W, H V]
     big_t: torch.Tensor = None
@@ -814,8 +816,10 @@ def convert_murulorn(cfg, tensors: dict, device="cpu", dtype=torch.bfloat16) -> 
             mix = ChannelDeltaWeights(big=big, n_big=big.shape[0],
                                       conv=torch.cat([f(p + "mix.q.conv"), f(p + "mix.k.conv"),
                                                       f(p + "mix.v.conv")]).contiguous(),
-                                      a_log=f(p + "mix.A_log"), dt_bias=f(p + "mix.dt_bias"), a2=f(p + "mix.a2"),
-                                      g2=f(p + "mix.g2"), norm=f(p + "mix.norm"), o=t(p + "mix.o"))
+                                      a_log=f(p + "mix.A_log"), dt_bias=f(p + "mix.dt_bias"),
+                                      ag2=torch.block_diag(f(p + "mix.a2"), f(p + "mix.g2")).contiguous(),
+                                      ra=tensors[p + "mix.a2"].shape[1], rg=tensors[p + "mix.g2"].shape[1],
+                                      norm=f(p + "mix.norm"), o=t(p + "mix.o"))
         _tile_fields(mix, ("big", "o"))
         layer = BracketLayer(norm1=gain(p + "norm1"), norm1b=gain(p + "norm1b"), mix=mix)
         fs = L.mlp

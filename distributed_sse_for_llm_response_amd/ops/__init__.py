@@ -283,4 +283,4 @@ from .layers import (conv_state, embed_rows, gate_math, gated_act, gated_head_no
                      latent_flash_ok, latent_flash_part_floats, latent_kv_write, logit_cap, lru_scan, matrix_scan, matrix_scan_chunked,
                      moe_ffn, moe_grouped, moe_router, moe_topk, norm_rope_rows, rms_mix, scalar_norm, sink_attention,
                      sink_flash_ok, stream_step, stream_mix, act_rows, moe_route, embed_pair_rows, add_norm_rows,
-                     token_gate_rows)
+                     token_gate_rows, token_side_rows, token_side_fits)

@@ -372,3 +372,26 @@ def token_gate_rows(x, ids, table, col0: int, out):
         torch.ops.dsse.token_gate_rows(x, ids, table, col0, out)
     else:
         lref.token_gate_rows(x, ids, table, col0, out)
+
+
+
+SIDE_FUSED_MAX_ROWS = 64   # steps of up to this many rows run a token input as one launch (each row's workgroup reads
+                           # both small weights from L2; prompt-sized steps amortise them in two GEMMs instead)
+
+
+def token_side_fits(rows: int, width: int, cols: int) -> bool:
+    """Steps that token_side_rows serves: decode-sized, the row and the gate's columns in 64 KB of LDS."""
+    return rows <= SIDE_FUSED_MAX_ROWS and (width + cols + 8) * 4 <= 64 * 1024
+
+
+def token_side_rows(y, nsum: int, g_add, resid, ids, table, col0: int, gate_w, proj_w, side_norm, g_out, eps: float,
+                    out=None, out32=None):
+    """A per-layer token input in ONE launch, for decode-sized steps: the pending add_norm_rows (y, nsum, g_add); the
+    gate g = gelu_tanh(gate_w x) * table[ids, col0 : col0 + F] on the stream rounded to the weights' type; the
+    back-projection proj_w g, RMS-normed, times side_norm, added to the stream; then out (element type; a column slice
+    is fine) = the stream normed with g_out (or itself), out32 the same unrounded."""
+    if _hip(resid):
+        torch.ops.dsse.token_side_rows(y, nsum, g_add, resid, ids, table, col0, gate_w, proj_w, side_norm, g_out, eps, out,
+                                       out32)
+    else:
+        lref.token_side_rows(y, nsum, g_add, resid, ids, table, col0, gate_w, proj_w, side_norm, g_out, eps, out, out32)

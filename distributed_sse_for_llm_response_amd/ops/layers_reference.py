@@ -499,3 +499,15 @@ def token_gate_rows(x, ids, table, col0, out):
     idx = ids[:x.shape[0]].long()
     idx = torch.where((idx >= 0) & (idx < table.shape[0]), idx, torch.zeros_like(idx))
     out.copy_((gelu_tanh(x.float()) * table[idx, col0:col0 + F].float()).to(out.dtype))
+
+
+def token_side_rows(y, nsum, g_add, resid, ids, table, col0, gate_w, proj_w, side_norm, g_out, eps, out, out32):
+    """A per-layer token input in one call: the pending add + norm; g = gelu_tanh(gate_w x) * table[ids, col0 : col0 + F]
+    on the stream rounded to the weights' type; resid += proj_w g, RMS-normed, times side_norm; then out = the stream
+    normed with g_out (or itself)."""
+    add_norm_rows(y, nsum, g_add, resid, None, eps, None, None)
+    F = gate_w.shape[0]
+    sg = resid.to(gate_w.dtype).float() @ gate_w.float().t()
+    sh = torch.empty(resid.shape[0], F, dtype=gate_w.dtype)
+    token_gate_rows(sg, ids, table, col0, sh)
+    add_norm_rows(sh.float() @ proj_w.float().t(), 1, side_norm, resid, g_out, eps, out, out32)

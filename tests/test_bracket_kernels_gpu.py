@@ -264,3 +264,48 @@ def test_delta_rule_under_a_per_channel_decay(H, G, D, V):
         ops.matrix_scan(c(q), c(k), c(v), c(decay), c(beta), st, c(qs), c(i32(ql)), c(i32(ctx)), c(i32(slot)), o, 1.0)
         close(o, o_ref, 2e-5)
         close(scan_state_plain(st), st_ref, 2e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("W,F,nsum", [(1, 1, 1), (19, 3, 2), (256, 24, 1), (2048, 64, 3), (1000, 20, 1)])
+def test_token_side_rows(dtype, W, F, nsum):
+    """The one-launch token input against its reference: with and without a pending add, a following norm, a strided
+    output and the unrounded copy."""
+    g = torch.Generator().manual_seed(14)
+    M, V = 6, 30
+    y, resid = torch.randn(M * nsum, W, generator=g), torch.randn(M, W, generator=g)
+    ga, go, sn = (torch.randn(W, generator=g) for _ in range(3))
+    gate_w = (torch.randn(F, W, generator=g) / math.sqrt(W)).to(dtype)
+    proj_w = (torch.randn(W, F, generator=g) / math.sqrt(F)).to(dtype)
+    table = torch.randn(V, 2 * F + 3, generator=g).to(dtype)
+    ids = i32(torch.randint(0, V, (M,), generator=g).tolist())
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    for use_y, use_go, use_out, use_32 in ((1, 1, 1, 1), (0, 0, 1, 0), (1, 0, 0, 0), (1, 1, 1, 0)):
+        r_ref = resid.clone()
+        wide_ref, o32_ref = torch.zeros(M, 2 * W + 8, dtype=dtype), torch.zeros(M, W)
+        lref.token_side_rows(y if use_y else None, nsum, ga if use_y else None, r_ref, ids, table, F + 1, gate_w, proj_w, sn,
+                             go if use_go else None, 1e-5, wide_ref[:, :W] if use_out else None, o32_ref if use_32 else None)
+        r = c(resid.clone())
+        wide, o32 = torch.zeros(M, 2 * W + 8, dtype=dtype, device=dev()), torch.zeros(M, W, device=dev())
+        ops.token_side_rows(c(y) if use_y else None, nsum, c(ga) if use_y else None, r, c(ids), c(table), F + 1, c(gate_w),
+                            c(proj_w), c(sn), c(go) if use_go else None, 1e-5, wide[:, :W] if use_out else None,
+                            o32 if use_32 else None)
+        close(r, r_ref, tol)
+        if use_out:
+            close(wide, wide_ref, tol)
+        if use_32:
+            close(o32, o32_ref, tol)
+    assert ops.token_side_fits(64, 8192, 256) and not ops.token_side_fits(65, 64, 8) and not ops.token_side_fits(4, 16384, 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1000, 16, 2048), (333, 64, 300), (40, 5, 256), (17, 1, 4100)])
+def test_many_rows_of_a_narrow_output(dtype, M, N, K):
+    """A router's logits or a few-column gate for a prompt: 16 x 16 output tiles with the K axis split over the waves."""
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(M, K + 3, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    ref = x[:, :K].float() @ w.float().t()
+    out = torch.zeros(M, N, device=dev())
+    ops.gemm_rm(c(x)[:, :K], c(w), out)
+    close(out, ref, 1e-5 if dtype == torch.float32 else 1e-2)

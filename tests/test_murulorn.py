@@ -672,7 +672,7 @@ def test_config_round_trip_and_registry(tmp_path):
     fam, cfg2, path = registry.resolve(str(tmp_path))
     assert fam.name == "murulorn" and cfg2.layers == cfg.layers and cfg2.width == cfg.width and path == str(tmp_path)
     w = registry.load_weights(fam, cfg2, path, device="cpu", dtype=torch.float32)
-    assert w.layers[1].mlp.up.shape == (6, 9, 72) and w.layers[1].mix.a2.shape == (4 * 6, 5) and w.layers[1].mix.g2.shape == (40, 3)
+    assert w.layers[1].mlp.up.shape == (6, 9, 72) and w.layers[1].mix.ag2.shape == (4 * 6 + 40, 5 + 3) and (w.layers[1].mix.ra, w.layers[1].mix.rg) == (5, 3)
     assert w.head is w.embed and w.bigram.shape == (38, 72) and w.loop_in.shape == (72, 144) and w.layers[2].side.col0 == 14
     assert torch.allclose(w.layers[0].norm1, 1.0 + weights["l0.norm1"].float())
     assert set(tensor_shapes(cfg)) == set(weights)

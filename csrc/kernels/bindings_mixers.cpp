@@ -652,7 +652,7 @@ void token_side_rows(const OptTensor& y, int64_t nsum, const OptTensor& g_add, T
   TORCH_CHECK(gate_w.scalar_type() == proj_w.scalar_type() && table.scalar_type() == gate_w.scalar_type(),
               "gate_w, proj_w and table share the element type");
   TORCH_CHECK(col0 >= 0 && col0 + p.F <= table.size(1) && ids.numel() >= p.M, "table must hold col0 + F columns, one id per row");
-  TORCH_CHECK((int64_t)(p.W + p.F + 8) * 4 <= 64 * 1024, "row too wide for the one-launch form");
+  TORCH_CHECK((int64_t)(p.W + p.F + 16) * 4 <= 64 * 1024, "row too wide for the one-launch form");
   p.f32 = elem(gate_w, "gate_w");
   p.resid = resid.data_ptr<float>();
   p.nsum = (int)nsum;

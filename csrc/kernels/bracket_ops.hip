@@ -181,38 +181,54 @@ __global__ __launch_bounds__(256) void token_gate_rows_kernel(const float* x, in
   }
 }
 
-// One workgroup per row.  The row lives in LDS: first the rounded stream (what the gate's projection reads), then the
-// back-projection's output.  A wave owns every fourth gate column (lanes stride over the width, 16-byte loads); a
-// thread owns every 256th channel of the back-projection (its weight row is F contiguous numbers).
+// One workgroup of sixteen waves per row: a decode step has few rows, so a row's work is spread as wide as one
+// workgroup goes.  The row lives in LDS: first the rounded stream (what the gate's projection reads), then the
+// back-projection's output.  A wave owns gate columns in groups of four (one pass over the stream row feeds four
+// independent sums, so four 16-byte loads are in flight per step); a thread owns every 1024th channel of the
+// back-projection (its weight row is F contiguous numbers: independent 16-byte loads).
+constexpr int kSideThreads = 1024;
+
+DEV float block_sum_wide(float v, float* red) {  // red holds one number per wave
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < nw; ++i) s += red[i];
+  return s;
+}
+
 template <typename T>
-__global__ __launch_bounds__(256) void token_side_rows_kernel(TokenSideParams p) {
+__global__ __launch_bounds__(kSideThreads) void token_side_rows_kernel(TokenSideParams p) {
   extern __shared__ float side_sm[];
   float* xs = side_sm;      // [W]
   float* gs = xs + p.W;     // [F]
-  float* red = gs + p.F;    // [4]
+  float* red = gs + p.F;    // [16]
   constexpr int VEC = sizeof(T) == 2 ? 8 : 4;
   const int64_t row = blockIdx.x;
   const int W = p.W, F = p.F;
+  const int nt = blockDim.x, nw = blockDim.x >> 6;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* resid = p.resid + row * W;
   if (p.y) {
     const float* y = p.y + row * p.nsum * W;
     float sy = 0.f;
-    for (int d = threadIdx.x; d < W; d += 256) {
+    for (int d = threadIdx.x; d < W; d += nt) {
       float v = 0.f;
       for (int s = 0; s < p.nsum; ++s) v += y[(int64_t)s * W + d];
       xs[d] = v;
       sy += v * v;
     }
-    sy = block_sum256(sy, red);
+    sy = block_sum_wide(sy, red);
     const float inv = 1.0f / sqrtf(sy / (float)W + p.eps);
-    for (int d = threadIdx.x; d < W; d += 256) {
+    for (int d = threadIdx.x; d < W; d += nt) {
       const float r = resid[d] + xs[d] * inv * p.g_add[d];
       resid[d] = r;
       xs[d] = (float)(T)r;
     }
   } else {
-    for (int d = threadIdx.x; d < W; d += 256) xs[d] = (float)(T)resid[d];
+    for (int d = threadIdx.x; d < W; d += nt) xs[d] = (float)(T)resid[d];
   }
   __syncthreads();
   int id = p.ids[row];
@@ -220,35 +236,51 @@ __global__ __launch_bounds__(256) void token_side_rows_kernel(TokenSideParams p)
   const T* trow = reinterpret_cast<const T*>(p.table) + (int64_t)id * p.ldt + p.col0;
   const T* gate_w = reinterpret_cast<const T*>(p.gate_w);
   const bool vw = W % VEC == 0;
-  for (int j = wave; j < F; j += 4) {
-    const T* gw = gate_w + (int64_t)j * W;
-    float s = 0.f;
+  for (int j0 = wave * 4; j0 < F; j0 += nw * 4) {
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    const T* gw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) gw[u] = gate_w + (int64_t)(j0 + u < F ? j0 + u : j0) * W;
     if (vw) {
       for (int d = lane * VEC; d < W; d += 64 * VEC) {
-        if constexpr (VEC == 8) {
-          const bf16x8 t = *reinterpret_cast<const bf16x8*>(gw + d);
+        float x[VEC];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) s += (float)t[e] * xs[d + e];
-        } else {
-          const f32x4 t = *reinterpret_cast<const f32x4*>(gw + d);
+        for (int e = 0; e < VEC; ++e) x[e] = xs[d + e];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) s += t[e] * xs[d + e];
+        for (int u = 0; u < 4; ++u) {
+          if constexpr (VEC == 8) {
+            const bf16x8 t = *reinterpret_cast<const bf16x8*>(gw[u] + d);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[u] += (float)t[e] * x[e];
+          } else {
+            const f32x4 t = *reinterpret_cast<const f32x4*>(gw[u] + d);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[u] += t[e] * x[e];
+          }
         }
       }
     } else {
-      for (int d = lane; d < W; d += 64) s += (float)gw[d] * xs[d];
+      for (int d = lane; d < W; d += 64) {
+        const float x = xs[d];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s[u] += (float)gw[u][d] * x;
+      }
     }
-    s = wave_sum(s);
-    if (lane == 0) gs[j] = (float)(T)(gelu_tanh_f(s) * (float)trow[j]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float t = wave_sum(s[u]);
+      if (lane == 0 && j0 + u < F) gs[j0 + u] = (float)(T)(gelu_tanh_f(t) * (float)trow[j0 + u]);
+    }
   }
   __syncthreads();  // the gate columns are complete, and nobody reads the rounded stream any more
   const T* proj_w = reinterpret_cast<const T*>(p.proj_w);
   const bool vf = F % VEC == 0;
   float sy = 0.f;
-  for (int d = threadIdx.x; d < W; d += 256) {
+  for (int d = threadIdx.x; d < W; d += nt) {
     const T* pw = proj_w + (int64_t)d * F;
     float v = 0.f;
     if (vf) {
+#pragma unroll 8
       for (int j = 0; j < F; j += VEC) {
         if constexpr (VEC == 8) {
           const bf16x8 t = *reinterpret_cast<const bf16x8*>(pw + j);
@@ -266,10 +298,10 @@ __global__ __launch_bounds__(256) void token_side_rows_kernel(TokenSideParams p)
     xs[d] = v;  // this thread's own channel: read back below by the same thread
     sy += v * v;
   }
-  sy = block_sum256(sy, red);
+  sy = block_sum_wide(sy, red);
   const float inv = 1.0f / sqrtf(sy / (float)W + p.eps);
   float ss = 0.f;
-  for (int d = threadIdx.x; d < W; d += 256) {
+  for (int d = threadIdx.x; d < W; d += nt) {
     const float r = resid[d] + xs[d] * inv * p.side_norm[d];
     resid[d] = r;
     xs[d] = r;
@@ -278,12 +310,12 @@ __global__ __launch_bounds__(256) void token_side_rows_kernel(TokenSideParams p)
   if (!p.out && !p.out32) return;  // uniform
   float inv2 = 1.0f;
   if (p.g_out) {
-    ss = block_sum256(ss, red);
+    ss = block_sum_wide(ss, red);
     inv2 = 1.0f / sqrtf(ss / (float)W + p.eps);
   }
   T* out = p.out ? reinterpret_cast<T*>(p.out) + row * p.ldo : nullptr;
   float* out32 = p.out32 ? p.out32 + row * W : nullptr;
-  for (int d = threadIdx.x; d < W; d += 256) {
+  for (int d = threadIdx.x; d < W; d += nt) {
     float r = xs[d];
     if (p.g_out) r = r * inv2 * p.g_out[d];
     if (out) out[d] = (T)r;
@@ -337,9 +369,10 @@ extern "C" hipError_t dsse_token_gate_rows(const float* x, int ldx, const int* i
 
 extern "C" hipError_t dsse_token_side_rows(const dsse::TokenSideParams* p, hipStream_t st) {
   if (p->M <= 0) return hipSuccess;
-  const size_t lds = (size_t)(p->W + p->F + 8) * sizeof(float);
+  const size_t lds = (size_t)(p->W + p->F + 16) * sizeof(float);
   if (p->nsum < 1 || (p->y && !p->g_add) || p->F < 1 || lds > 64 * 1024) return hipErrorInvalidValue;
-  if (p->f32) hipLaunchKernelGGL(dsse::token_side_rows_kernel<float>, dim3(p->M), dim3(256), lds, st, *p);
-  else hipLaunchKernelGGL(dsse::token_side_rows_kernel<bf16>, dim3(p->M), dim3(256), lds, st, *p);
+  const dim3 block(dsse::kSideThreads);
+  if (p->f32) hipLaunchKernelGGL(dsse::token_side_rows_kernel<float>, dim3(p->M), block, lds, st, *p);
+  else hipLaunchKernelGGL(dsse::token_side_rows_kernel<bf16>, dim3(p->M), block, lds, st, *p);
   return hipGetLastError();
 }

@@ -86,10 +86,12 @@ __global__ __launch_bounds__(256) void gemm_rm_kernel(GemmRmParams p) {
 // (k-steps w, w + 4, ...), meeting in LDS.  Four times the workgroups of a 16 x 64 tile and a quarter of the dependent
 // k-steps per wave: these launches are latency-bound, not bandwidth-bound -- a narrow output leaves the 64 x 64 tiles
 // of the general kernel a handful of workgroups that each walk the whole K axis.
-template <typename T>
-__global__ __launch_bounds__(256) void gemm_rm_skinny_kernel(GemmRmParams p) {
+// NW waves per workgroup: four, or sixteen when the launch has few tiles and a long K axis (a router's logits for a
+// decode step are ONE tile: sixteen waves walk a sixteenth of K each instead of four a quarter).
+template <typename T, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_rm_skinny_kernel(GemmRmParams p) {
   using F = Frag<T>;
-  __shared__ float red[4 * 4 * 64];
+  __shared__ float red[NW * 4 * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int col0 = blockIdx.x * 16, row0 = blockIdx.y * 16;
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(256) void gemm_rm_skinny_kernel(GemmRmParams p) {
   const T* wr = W + (int64_t)(wv ? col0 + r : 0) * p.ldw;
   const bool vx = p.vecx != 0, vw = p.vecw != 0;
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = wave * F::KS; k0 < p.K; k0 += 4 * F::KS) {
+  for (int k0 = wave * F::KS; k0 < p.K; k0 += NW * F::KS) {
     const int k = k0 + F::PER * g;
     acc = mma(load_frag<T>(xr, k, p.K, xv, vx), load_frag<T>(wr, k, p.K, wv, vw), acc);
   }
@@ -117,7 +119,9 @@ __global__ __launch_bounds__(256) void gemm_rm_skinny_kernel(GemmRmParams p) {
   for (int e = 0; e < 4; ++e) {
     const int row = row0 + 4 * g + e;
     if (row >= p.M) continue;
-    float v = red[e * 64 + lane] + red[(4 + e) * 64 + lane] + red[(8 + e) * 64 + lane] + red[(12 + e) * 64 + lane] + bv;
+    float v = bv;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += red[(4 * w + e) * 64 + lane];
     if (p.act == 1) v = gelu_tanh(v);
     const int64_t o = (int64_t)z * p.obs + (int64_t)row * p.ldo + col;
     if (p.out_f32) reinterpret_cast<float*>(p.out)[o] = v;
@@ -135,7 +139,11 @@ hipError_t launch(const GemmRmParams& p, hipStream_t st) {
 template <typename T>
 hipError_t dispatch(const GemmRmParams& p, hipStream_t st) {
   if (p.M <= 16 || (p.N <= 64 && p.K >= 256)) {
-    hipLaunchKernelGGL(gemm_rm_skinny_kernel<T>, dim3((p.N + 15) / 16, (p.M + 15) / 16, p.batch), dim3(256), 0, st, p);
+    const dim3 grid((p.N + 15) / 16, (p.M + 15) / 16, p.batch);
+    if ((int64_t)grid.x * grid.y * grid.z <= 256 && p.K >= 64 * Frag<T>::KS)
+      hipLaunchKernelGGL((gemm_rm_skinny_kernel<T, 16>), grid, dim3(1024), 0, st, p);
+    else
+      hipLaunchKernelGGL((gemm_rm_skinny_kernel<T, 4>), grid, dim3(256), 0, st, p);
     return hipGetLastError();
   }
   if (p.M >= 256 && p.N >= 256) return launch<T, 4, 4, 2, 2>(p, st);

@@ -879,7 +879,7 @@ class LayeredRunner(RunnerBase):
 
     def _channel_delta_bracket(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
         """Gated delta rule with a decay per head and key channel: ONE fused GEMM [q | k | v | b | a1 | g1] (fp32 out)
-        -> conv_state over q | k | v (SiLU; slot tail) -> unit q, k per head -> the decay's and the gate's second
+        -> conv_state over q | k | v (SiLU; slot tail) -> unit q, k per head (the query's dim^-1/2 rides in the scan) -> the decay's and the gate's second
         projections in fp32 as one block-diagonal product -> gate_math (one rate per head, one bias per head and channel) -> matrix_scan (delta rule
         with per-channel decay; slot state) -> per-head RMS norm times the sigmoid gate -> output GEMM."""
         H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
@@ -891,8 +891,8 @@ class LayeredRunner(RunnerBase):
             ops.conv_state(big[:, :C], Lw.conv, None, self.state.tail.get(ri), g["qs"], g["ql"], g["ctx"], g["ss"], cv,
                            None, None, 1, g["qt"] == 1)
         q, k, v = self._cols(cv, 0, G, D), self._cols(cv, G * D, G, D), self._cols(cv, 2 * G * D, H, V)
-        ops.norm_rope_rows(q, None, pos, None, q, None, 2, UNIT_EPS, D ** -0.5)
-        ops.norm_rope_rows(k, None, pos, None, k, None, 2, UNIT_EPS, 1.0)
+        qk = self._cols(cv, 0, 2 * G, D)   # q and k heads side by side: one launch makes them unit vectors
+        ops.norm_rope_rows(qk, None, pos, None, qk, None, 2, UNIT_EPS, 1.0)
         beta = big[:, C:C + H]
         ops.gate_math(beta, 1)
         zz = d["z"][:M * H * (D + V)].view(M, H * (D + V))
@@ -902,7 +902,7 @@ class LayeredRunner(RunnerBase):
         o = d["o"][:M * H * V].view(M, H, V)
         for g in groups:
             ops.matrix_scan(q, k, v, z.unflatten(1, (H, D)), beta, self.state.state[ri], g["qs"], g["ql"], g["ctx"],
-                            g["ss"], o, 1.0)
+                            g["ss"], o, D ** -0.5)
         ao = d["ao"][:M * H * V].view(M, H * V)
         ops.gated_head_norm(o, Lw.norm, gz, self.cfg.eps, ao, 1)
         self._lin(ao, Lw.o, Lw.o_t, d["y"])

@@ -381,7 +381,7 @@ SIDE_FUSED_MAX_ROWS = 64   # steps of up to this many rows run a token input as 
 
 def token_side_fits(rows: int, width: int, cols: int) -> bool:
     """Steps that token_side_rows serves: decode-sized, the row and the gate's columns in 64 KB of LDS."""
-    return rows <= SIDE_FUSED_MAX_ROWS and (width + cols + 8) * 4 <= 64 * 1024
+    return rows <= SIDE_FUSED_MAX_ROWS and (width + cols + 16) * 4 <= 64 * 1024
 
 
 def token_side_rows(y, nsum: int, g_add, resid, ids, table, col0: int, gate_w, proj_w, side_norm, g_out, eps: float,

@@ -1,7 +1,8 @@
-"""Forward passes of configuration-driven designs (models/muderax.py, models/surodra.py, models/dironex.py) on the
-layer-mechanism kernels (ops/layers.py).  Three block styles share the runner: sandwich norms on a sublayer's output
-(Muderax, described first), pre-norm blocks around matrix-state mixers (Surodra, described after it) and pre-norm
-blocks on several residual streams (Dironex, described last).
+"""Forward passes of configuration-driven designs (models/muderax.py, models/surodra.py, models/dironex.py,
+models/murulorn.py) on the layer-mechanism kernels (ops/layers.py).  Four block styles share the runner: sandwich
+norms on a sublayer's output (Muderax, described first), pre-norm blocks around matrix-state mixers (Surodra,
+described after it), pre-norm blocks on several residual streams (Dironex) and blocks with a norm before and after
+each sublayer plus a per-layer token input (Murulorn, described last).
 
 A step is a set of packed rows -- the B decode slots first (one row each, state on the device as in ModelRunner), then
 the rows of prompt portions -- that walk the layer list once:
@@ -54,6 +55,30 @@ The multi-stream walk (`_stream_layers`) also goes over layer runs; a row carrie
                             (group-limited sigmoid routing) -> moe_grouped without a gate (squared ReLU), per-slot outputs
                             summed inside the next stream_mix
     head                    stream_mix (last write-back, sum of the streams) -> RMS norm -> head GEMM
+
+The bracket-norm walk (`_bracket_layers`) also goes over layer runs:
+
+    embed_pair_rows         stream = embed[token] + pair[hash(previous token, token)] (the table's last row at position
+                            0); the embedding output once more, rounded, beside the stream's place in [stream | x0]
+    add_norm_rows           between sublayers: stream += rms-norm(finished sublayer) * gain; xb = rms-norm(stream) * gain
+                            of the next one (also fp32 for a router), or the rounded stream
+    loop pass               stream <- W_in [stream | x0] (one GEMM on the rounded pair) before the pass's first layer
+    attention layer         ONE fused GEMM [q | k | v | g] -> norm_rope_rows (whole-row RMS + rotation: q to a buffer, k
+                            into the run's pages; v: RMS per head + rotation over its whole width into the pages) ->
+                            sink_attention with capped scores, the head's sum turned back by the row's position, sigmoid
+                            gate -> output GEMM
+    channel-delta layer     ONE fused GEMM [q | k | v | b | a1 | g1] -> conv_state (SiLU; slot tail) -> unit q | k ->
+                            block-diagonal fp32 GEMM [a2 0; 0 g2] -> gate_math (rate per head, bias per head and channel)
+                            -> matrix_scan (delta rule, per-channel decay; slot state) -> gated_head_norm (sigmoid) ->
+                            output GEMM
+    feed-forward            up GEMM -> act_rows (squared ReLU) -> down GEMM; or router GEMM in fp32 on the fp32 row ->
+                            moe_route (softmax scores, group maxima) -> moe_grouped without a gate
+    token input             steps of up to 64 rows: token_side_rows, one launch that also writes the next sublayer's
+                            input; larger steps: rounding, gate GEMM, token_gate_rows, back-projection GEMM
+    head                    add_norm_rows (final norm) -> GEMM on the embedding table
+
+A decode row's token becomes its slot's previous token inside embed_pair_rows (the captured graph carries it); prompt
+portions bring each row's predecessor with them (PrefillSeq.prev_token for the first row).
 
 The residual stream, norms, scores, router and recurrence are fp32 in both element types; ``dtype=torch.float32`` runs
 the projections in true fp32 as well (the exact mode).  The cache is paged with the engine's block tables and
@@ -879,8 +904,9 @@ class LayeredRunner(RunnerBase):
 
     def _channel_delta_bracket(self, ri: int, m, Lw, M: int, d: dict, pos, slots, groups: list) -> None:
         """Gated delta rule with a decay per head and key channel: ONE fused GEMM [q | k | v | b | a1 | g1] (fp32 out)
-        -> conv_state over q | k | v (SiLU; slot tail) -> unit q, k per head (the query's dim^-1/2 rides in the scan) -> the decay's and the gate's second
-        projections in fp32 as one block-diagonal product -> gate_math (one rate per head, one bias per head and channel) -> matrix_scan (delta rule
+        -> conv_state over q | k | v (SiLU; slot tail) -> unit q, k per head in one launch (the query's dim^-1/2
+        rides in the scan) -> the decay's and the gate's second projections in fp32 as one block-diagonal product
+        -> gate_math (one rate per head, one bias per head and channel) -> matrix_scan (delta rule
         with per-channel decay; slot state) -> per-head RMS norm times the sigmoid gate -> output GEMM."""
         H, G, D, V = m.heads, m.kv_heads, m.dim, m.vdim
         C = 2 * G * D + H * V
